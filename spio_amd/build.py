@@ -1,0 +1,80 @@
+"""Builds the native pieces of the package in-tree.
+
+`build_native()` compiles csrc/spio_hip.cpp into csrc/libspio_hip.so with the
+host C++ compiler.  The library has no link-time dependency on the HIP
+runtime (it binds it with dlopen), so it builds on machines without a GPU.
+
+`check_kernels()` compiles every HIP kernel source for gfx950 with hipcc for
+a list of representative shape specialisations; at run time the same sources
+are specialised per shape with hipRTC instead.
+"""
+
+import os
+import shutil
+import subprocess
+import sys
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC_DIR = os.path.join(_HERE, "csrc")
+REPO_INCLUDE_DIR = os.path.join(os.path.dirname(_HERE), "include")
+LIB_PATH = os.path.join(CSRC_DIR, "libspio_hip.so")
+ROCM_HOME = os.environ.get("ROCM_PATH") or os.environ.get("ROCM_HOME") or "/opt/rocm"
+
+# hipcc flags shared by every device compilation of this package.
+HIPCC_DEVICE_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-Xclang",
+    "-target-feature",
+    "-Xclang",
+    "-packed-fp32-ops",
+]
+
+
+def _include_dir() -> str:
+    """Directory holding spio_hip.h (repo layout or a copy inside csrc)."""
+    if os.path.exists(os.path.join(REPO_INCLUDE_DIR, "spio_hip.h")):
+        return REPO_INCLUDE_DIR
+    return CSRC_DIR
+
+
+def build_native(force: bool = True, verbose: bool = False) -> str:
+    """Compile libspio_hip.so; returns its path."""
+    src = os.path.join(CSRC_DIR, "spio_hip.cpp")
+    if not force and os.path.exists(LIB_PATH) and os.path.getmtime(LIB_PATH) >= os.path.getmtime(src):
+        return LIB_PATH
+    cxx = os.environ.get("CXX") or shutil.which("g++") or shutil.which("c++")
+    if cxx is None:
+        raise RuntimeError("no host C++ compiler found to build libspio_hip.so")
+    tmp = LIB_PATH + f".tmp{os.getpid()}"
+    cmd = [
+        cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall",
+        f"-I{_include_dir()}", f"-I{os.path.join(ROCM_HOME, 'include')}",
+        "-o", tmp, src, "-ldl", "-lpthread",
+    ]  # fmt: skip
+    if verbose:
+        print(" ".join(cmd))
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"building libspio_hip.so failed:\n{proc.stdout}\n{proc.stderr}")
+    os.replace(tmp, LIB_PATH)
+    return LIB_PATH
+
+
+def hipcc_compile_check(source_path: str, defines: dict, out_dir: str, tag: str) -> str:
+    """Compile one kernel source to a gfx950 code object with hipcc."""
+    hipcc = shutil.which("hipcc") or os.path.join(ROCM_HOME, "bin", "hipcc")
+    out = os.path.join(out_dir, f"{tag}.co")
+    cmd = [hipcc, "--genco", *HIPCC_DEVICE_FLAGS, f"-I{CSRC_DIR}"]
+    cmd += [f"-D{k}={v}" for k, v in defines.items()]
+    cmd += ["-o", out, source_path]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {tag}:\n{' '.join(cmd)}\n{proc.stderr}")
+    return out
+
+
+if __name__ == "__main__":
+    print(build_native(verbose=True))
+    sys.exit(0)

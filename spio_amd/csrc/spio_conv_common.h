@@ -1,0 +1,86 @@
+// Shared definitions for the grouped-width-8 convolution kernels (gfx950).
+//
+// Every kernel of this directory is specialised at compile time: the shape of
+// one convolution and the tile configuration arrive as SPIO_* macros, either
+// from hipRTC options at run time or from -D flags of an offline hipcc build.
+// Kernels therefore take only pointers, as the reference's kernels do
+// (spio/src/conv2d_gw8.cu:10-12, spio/src/conv2d_gw8_wgrad.cu:10-12).
+//
+// Memory layouts (physical):
+//   activations  [N][H][W][C]      fp16   (NCHW tensors with channels_last strides)
+//   weights      [K][R][S][8]      fp16   ([K,8,R,S] tensors with channels_last strides)
+//   bias         [K]               fp32
+//   grad_weight  [K][R][S][8]      fp32
+// A group is 8 consecutive channels: 16 bytes of one pixel.
+#ifndef SPIO_CONV_COMMON_H
+#define SPIO_CONV_COMMON_H
+
+#ifndef SPIO_N
+#error "shape macros (SPIO_N, SPIO_C, SPIO_H, SPIO_W, SPIO_R, SPIO_S, SPIO_PY, SPIO_PX) are required"
+#endif
+
+typedef _Float16 spio_half;
+typedef _Float16 spio_half2 __attribute__((ext_vector_type(2)));
+typedef _Float16 spio_half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 spio_half8 __attribute__((ext_vector_type(8)));
+typedef float spio_float4 __attribute__((ext_vector_type(4)));
+typedef unsigned int spio_uint2 __attribute__((ext_vector_type(2)));
+typedef unsigned int spio_uint4 __attribute__((ext_vector_type(4)));
+typedef short spio_short4 __attribute__((ext_vector_type(4)));
+
+namespace spio {
+
+// The convolution as the user states it (forward orientation).
+constexpr int kN = SPIO_N;
+constexpr int kC = SPIO_C;
+constexpr int kH = SPIO_H;
+constexpr int kW = SPIO_W;
+constexpr int kR = SPIO_R;
+constexpr int kS = SPIO_S;
+constexpr int kPadY = SPIO_PY;
+constexpr int kPadX = SPIO_PX;
+constexpr int kP = kH + 2 * kPadY - kR + 1;
+constexpr int kQ = kW + 2 * kPadX - kS + 1;
+constexpr int kGroups = kC / 8;
+
+static_assert(kC % 8 == 0, "channels must be a multiple of the group width 8");
+static_assert(kP > 0 && kQ > 0, "empty output");
+
+// The kernels use compiler builtins only, so they compile identically under
+// hipRTC and under an offline hipcc build without any runtime header.
+#define SPIO_DEVICE __device__ inline __attribute__((always_inline))
+#define SPIO_LAUNCH_BOUNDS(threads) __attribute__((amdgpu_flat_work_group_size(threads, threads)))
+
+SPIO_DEVICE int imin(int a, int b) { return a < b ? a : b; }
+SPIO_DEVICE int imax(int a, int b) { return a > b ? a : b; }
+SPIO_DEVICE int thread_id() { return (int)__builtin_amdgcn_workitem_id_x(); }
+SPIO_DEVICE int block_id() { return (int)__builtin_amdgcn_workgroup_id_x(); }
+
+// Workgroup barrier with LDS/global visibility among the waves of the group.
+SPIO_DEVICE void block_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+}
+
+// Device-scope fp32 add without a return value.
+SPIO_DEVICE void atomic_add_f32(float* address, float value) {
+    __hip_atomic_fetch_add(address, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Bit-cast helpers between the 16-byte vector views of one (pixel, group).
+union Pack16 {
+    spio_uint4 u;
+    spio_half8 h;
+    spio_half4 h4[2];
+};
+
+union Pack8 {
+    spio_uint2 u;
+    spio_half4 h;
+    spio_short4 s;
+};
+
+}  // namespace spio
+
+#endif  // SPIO_CONV_COMMON_H

@@ -1,0 +1,3 @@
+"""Functional interface: the `spio::conv2d_gw8` custom operators."""
+
+from .conv2d_gw8_function import conv2d_gw8, conv2d_gw8_backward_op

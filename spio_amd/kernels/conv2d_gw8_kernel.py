@@ -1,0 +1,199 @@
+"""Forward / data-gradient kernel family of conv2d_gw8.
+
+Reference: spio/kernels/conv2d_gw8_kernel.py:30-238 (`Conv2dGw8Config`,
+`_get_configs`, `_get_kernel_spec`; `igrad=True` selects the data gradient,
+which reuses the forward kernel with the flipped, group-transposed filter and
+padding (R-1-py, S-1-px), :73-83).  The tile configuration is re-designed for
+CDNA4: see csrc/conv2d_gw8_mfma.hip for what the fields mean on the device.
+"""
+
+from dataclasses import dataclass
+from math import gcd
+from typing import Dict, List
+
+import torch
+
+from ..util.math import divup
+from .conv2d_gw8_params import Conv2dGw8Params
+from .conv2d_stats import Conv2dStats
+from .kernel import KernelSpec
+from .kernel_factory import KernelFactory
+from .launch_params import LaunchParams
+
+MFMA_SOURCE = "conv2d_gw8_mfma.hip"
+DIRECT_SOURCE = "conv2d_gw8_direct.hip"
+
+MAX_WAVES = 16
+MAX_LDS_BYTES = 64 * 1024
+MAX_LOADS_PER_THREAD = 8
+MAX_ACCUMULATORS = 16
+MAX_CONFIGS = 28
+
+
+@dataclass(frozen=True)
+class Conv2dGw8Config:
+    """Tile configuration of the forward / data-gradient kernel.
+
+    Attributes:
+        groups: channel groups per workgroup (one wave per group and split).
+        block_p: output rows per workgroup.
+        block_n: images whose rows are laid side by side in one staged row.
+        split: waves sharing the 16-pixel tiles of one group.
+        prefetch: rows of global loads in flight ahead of the computed row.
+        variant: "mfma" (row-streaming MFMA kernel) or "direct" (one thread per
+            output pixel-group; any shape).
+    """
+
+    groups: int = 8
+    block_p: int = 16
+    block_n: int = 1
+    split: int = 1
+    prefetch: int = 2
+    variant: str = "mfma"
+
+
+def direction_geometry(params: Conv2dGw8Params, igrad: bool) -> Dict[str, int]:
+    """Source/destination extents and effective padding of one direction."""
+    if igrad:
+        return dict(SH=params.p, SW=params.q, DH=params.h, DW=params.w,
+                    EPY=params.transpose_padding_h, EPX=params.transpose_padding_w)  # fmt: skip
+    return dict(SH=params.h, SW=params.w, DH=params.p, DW=params.q,
+                EPY=params.padding_h, EPX=params.padding_w)  # fmt: skip
+
+
+def mfma_geometry(params: Conv2dGw8Params, config: Conv2dGw8Config, igrad: bool) -> Dict[str, int]:
+    """Host mirror of the compile-time constants of conv2d_gw8_mfma.hip."""
+    d = direction_geometry(params, igrad)
+    r, s = params.r, params.s
+    gb, bp, nb, ts, pf = config.groups, config.block_p, config.block_n, config.split, config.prefetch
+    ns = 2 * ((r + 1) // 2)
+    kb = (s + 3) // 4
+    wpi = d["DW"] + s - 1
+    f = nb * wpi
+    wt = divup(f - s + 1, 16)
+    fp = 16 * wt + 4 * kb - 1
+    gs = fp + ((9 - fp % 16) + 16) % 16
+    threads = 64 * gb * ts
+    ostride = gb * 16 + 16
+    lds = 2 * gb * gs * 16 + 2 * 16 * wt * ostride
+    d.update(
+        NS=ns, NACC=ns // 2, KB=kb, WPI=wpi, F=f, WT=wt, TPW=divup(wt, ts), GS=gs,
+        THREADS=threads, LDS_BYTES=lds, LPT=divup(f * gb, threads),
+        SPT=divup(nb * d["DW"] * gb, threads),
+        GBLKS=divup(params.groups, gb), PBLKS=divup(d["DH"], bp), NBLKS=divup(params.n, nb),
+        STEPS=bp + r - 1, UNROLL=ns // gcd(ns, pf) * pf,
+    )  # fmt: skip
+    d["NUM_BLOCKS"] = d["GBLKS"] * d["PBLKS"] * d["NBLKS"]
+    return d
+
+
+def _mfma_config_is_legal(params, config, igrad) -> bool:
+    g = mfma_geometry(params, config, igrad)
+    return (
+        config.groups * config.split <= MAX_WAVES
+        and config.split <= g["WT"]
+        and config.block_n <= max(params.n, 1)
+        and config.block_p <= g["DH"]
+        and g["LDS_BYTES"] <= MAX_LDS_BYTES
+        and g["LPT"] <= MAX_LOADS_PER_THREAD
+        and g["TPW"] * g["NACC"] <= MAX_ACCUMULATORS
+        and config.prefetch >= 2
+        and g["UNROLL"] <= 12
+    )
+
+
+def _mfma_score(params, config, igrad, num_cus: int) -> float:
+    """Rough relative cost used only to order (and cap) the sweep."""
+    g = mfma_geometry(params, config, igrad)
+    halo_rows = (config.block_p + params.r - 1) / config.block_p
+    useful = config.block_n * g["DW"]
+    tile_eff = useful / (16.0 * g["WT"])
+    group_eff = params.groups / (g["GBLKS"] * config.groups)
+    # Workgroups per CU limited by LDS and by 2048 threads.
+    per_cu = max(1, min(160 * 1024 // g["LDS_BYTES"], 2048 // g["THREADS"], 8))
+    slots = num_cus * per_cu
+    waves_of_blocks = divup(g["NUM_BLOCKS"], slots)
+    quant = waves_of_blocks * slots / g["NUM_BLOCKS"]
+    return halo_rows ** 0.5 * quant / (tile_eff * group_eff)
+
+
+def _get_configs(params: Conv2dGw8Params, device_attr=None, igrad: bool = False) -> List[Conv2dGw8Config]:
+    """Legal configurations, most promising first; the direct kernel is always last."""
+    d = direction_geometry(params, igrad)
+    num_cus = getattr(device_attr, "multiprocessor_count", 256) or 256
+    G = params.groups
+    group_choices = sorted({g for g in (4, 8, 16, G) if g <= min(G, MAX_WAVES)}) or [min(G, MAX_WAVES)]
+    row_choices = sorted({bp for bp in (2, 4, 7, 8, 14, 16, 28, 32, 56, d["DH"]) if bp <= d["DH"]})
+    found = []
+    for gb in group_choices:
+        for nb in (1, 2, 4, 8):
+            for ts in (1, 2, 4):
+                for bp in row_choices:
+                    cfg = Conv2dGw8Config(groups=gb, block_p=bp, block_n=nb, split=ts)
+                    if _mfma_config_is_legal(params, cfg, igrad):
+                        found.append((_mfma_score(params, cfg, igrad, num_cus), cfg))
+    found.sort(key=lambda sc: sc[0])
+    configs = [cfg for _, cfg in found[:MAX_CONFIGS]]
+    configs.append(Conv2dGw8Config(groups=1, block_p=1, block_n=1, split=1, variant="direct"))
+    return configs
+
+
+def _shape_defines(params: Conv2dGw8Params) -> Dict[str, object]:
+    return {
+        "SPIO_N": params.n, "SPIO_C": params.c, "SPIO_H": params.h, "SPIO_W": params.w,
+        "SPIO_R": params.r, "SPIO_S": params.s,
+        "SPIO_PY": params.padding_h, "SPIO_PX": params.padding_w,
+    }  # fmt: skip
+
+
+def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8Config, _device_attr=None,
+                     igrad: bool = False) -> KernelSpec:  # fmt: skip
+    """Macros and launch geometry for one (params, config, direction)."""
+    params.validate()
+    defines = _shape_defines(params)
+    defines["SPIO_IGRAD"] = int(igrad)
+    defines["SPIO_HAS_BIAS"] = int(params.has_bias and not igrad)
+    if config.variant == "direct":
+        d = direction_geometry(params, igrad)
+        threads = 256
+        defines["SPIO_BLOCK_THREADS"] = threads
+        total = params.n * d["DH"] * d["DW"] * params.groups
+        return KernelSpec(defines, LaunchParams(grid=divup(total, threads), block=threads), DIRECT_SOURCE)
+    if config.variant != "mfma":
+        raise ValueError(f"unknown kernel variant {config.variant!r}")
+    assert _mfma_config_is_legal(params, config, igrad), f"illegal configuration {config} for {params}"
+    g = mfma_geometry(params, config, igrad)
+    defines.update(
+        SPIO_GB=config.groups, SPIO_BP=config.block_p, SPIO_NB=config.block_n,
+        SPIO_TS=config.split, SPIO_PF=config.prefetch,
+    )  # fmt: skip
+    return KernelSpec(
+        defines, LaunchParams(grid=g["NUM_BLOCKS"], block=g["THREADS"]), MFMA_SOURCE, notes=g
+    )
+
+
+def _get_kernel_name(igrad: bool = False) -> str:
+    return "spio_conv2d_gw8_dgrad" if igrad else "spio_conv2d_gw8_fprop"
+
+
+def _make_test_args(params: Conv2dGw8Params, device, igrad: bool = False):
+    """Synthetic (dst, src, weight, bias) for timing."""
+    cl = torch.channels_last
+    x = torch.randn(params.input_shape, device=device, dtype=torch.float16).contiguous(memory_format=cl)
+    y = torch.randn(params.output_shape, device=device, dtype=torch.float16).contiguous(memory_format=cl)
+    w = (torch.randn(params.weight_shape, device=device, dtype=torch.float16) * 0.1).contiguous(memory_format=cl)
+    if igrad:
+        return (x, y, w, None)
+    bias = torch.randn(params.bias_shape, device=device, dtype=torch.float32) if params.has_bias else None
+    return (y, x, w, bias)
+
+
+conv2d_gw8_kernel_factory = KernelFactory(
+    Conv2dGw8Params,
+    Conv2dGw8Config,
+    Conv2dStats,
+    kernel_name=_get_kernel_name,
+    configs=_get_configs,
+    kernel_spec=_get_kernel_spec,
+    make_test_args=_make_test_args,
+)

@@ -1,0 +1,134 @@
+"""One shape-specialised GPU kernel: compile, load, launch.
+
+Reference: spio/kernels/kernel.py:22-174.  The reference generates a C++
+header of typed dimensions per kernel; here every constant is a `-D` macro
+(`KernelSpec.defines`) and the source is one of the HIP files in csrc/.
+"""
+
+from dataclasses import dataclass, field
+from typing import Dict, Optional
+
+import torch
+
+from ..compiler.compile_kernel import compile_kernel, load_kernel
+from ..compiler import flags
+from ..util.memory_format import check_channels_last
+from .launch_params import LaunchParams
+
+
+@dataclass
+class KernelSpec:
+    """Everything that specialises one kernel build and its launch.
+
+    Attributes:
+        defines: macro name -> value for the compilation.
+        launch_params: grid, block and dynamic LDS bytes.
+        source_file: HIP source inside csrc/.
+        max_dynamic_lds: when set, the kernel's dynamic LDS limit is raised to it.
+    """
+
+    defines: Dict[str, object]
+    launch_params: LaunchParams
+    source_file: str
+    max_dynamic_lds: Optional[int] = None
+    notes: Dict[str, object] = field(default_factory=dict)
+
+
+class Kernel:
+    """A compiled kernel bound to one device.  Made by KernelFactory.make_kernel."""
+
+    def __init__(self, kernel_name, kernel_spec: KernelSpec, params=None, config=None,
+                 args_checker=check_channels_last):  # fmt: skip
+        self.kernel_name = kernel_name
+        self.kernel_spec = kernel_spec
+        self.params = params
+        self.config = config
+        self.args_checker = args_checker
+        self.code: Optional[bytes] = None
+        self.module = None
+        self.function = None
+        self.device_ordinal: Optional[int] = None
+
+    @property
+    def kernel_source_file(self) -> str:
+        return self.kernel_spec.source_file
+
+    @property
+    def defines(self) -> Dict[str, object]:
+        d = dict(self.kernel_spec.defines)
+        d["SPIO_KERNEL_NAME"] = self.kernel_name
+        return d
+
+    def compile(self):
+        """JIT-compile the specialised source to a code object."""
+        self.code = compile_kernel(
+            self.kernel_source_file, self.defines,
+            debug=flags.debug.get(), lineinfo=flags.lineinfo.get(),
+        )  # fmt: skip
+
+    def load(self, device_ordinal: int = 0, clear_code: bool = True):
+        """Load the code object on a device and resolve the kernel symbol."""
+        if self.code is None:
+            raise ValueError(f"Kernel {self.kernel_name} has not been compiled")
+        self.module, self.function = load_kernel(self.kernel_name, self.code, device_ordinal)
+        self.device_ordinal = device_ordinal
+        if self.kernel_spec.max_dynamic_lds:
+            self.function.set_max_dynamic_lds(self.kernel_spec.max_dynamic_lds)
+        if clear_code:
+            self.code = None
+
+    def unload(self):
+        """Drop the module; load() may be called again if the code was kept."""
+        if self.module is not None:
+            self.module.unload()
+            self.module = None
+        self.function = None
+
+    def _prepare(self, args):
+        if self.function is None:
+            raise ValueError("kernel is not loaded")
+        if self.args_checker is not None:
+            self.args_checker(args)
+        device = None
+        for a in args:
+            if isinstance(a, torch.Tensor) and a.numel() > 0:
+                if device is None:
+                    device = a.device
+                assert a.device == device, "Not all tensor arguments are on the same device"
+        if device is None or device.type != "cuda":
+            raise ValueError("kernel arguments must be GPU tensors")
+        return device, [a.detach() if isinstance(a, torch.Tensor) else a for a in args]
+
+    def launch(self, *args):
+        """Asynchronous launch on torch's current stream of the arguments' device."""
+        try:
+            device, kargs = self._prepare(args)
+            lp = self.kernel_spec.launch_params
+            stream = torch.cuda.current_stream(device).cuda_stream
+            self.function.launch(lp.grid, lp.block, kargs, lp.shared_mem_bytes, stream)
+        except Exception as e:
+            raise ValueError(f"Error in kernel {self}") from e
+
+    def time(self, arg_sets, warmup: int = 3, iters: int = 20) -> float:
+        """Average milliseconds per launch, HIP events on torch's current stream."""
+        device = None
+        prepared = []
+        for args in arg_sets:
+            device, kargs = self._prepare(args)
+            prepared.append(kargs)
+        lp = self.kernel_spec.launch_params
+        stream = torch.cuda.current_stream(device).cuda_stream
+        return self.function.launch_timed(
+            lp.grid, lp.block, prepared, lp.shared_mem_bytes, stream, warmup, iters
+        )
+
+    def __call__(self, *args):
+        self.launch(*args)
+
+    def __repr__(self) -> str:
+        return f"{self.kernel_name} {self.config}"
+
+
+def get_full_kernel_name(kernel_name: str, params) -> str:
+    """`<kernel>__<params.encode()>` (reference: kernel.py:160-163)."""
+    return f"{kernel_name}__{params.encode()}"

@@ -1,0 +1,28 @@
+"""Cache keys (reference: spio/kernels/kernel_key.py:13-34)."""
+
+from dataclasses import dataclass
+from typing import Any, Tuple
+
+
+@dataclass(frozen=True)
+class KernelKey:
+    """Key of a kernel in a KernelCache."""
+
+    device_ordinal: int
+    params: Any
+
+
+@dataclass(frozen=True)
+class KernelParams:
+    """One kernel request captured by KernelParamsLogger."""
+
+    kernel_cache: Any
+    kernel_factory: Any
+    params: Any
+    device: Any
+    kernel_kwargs: Tuple[Tuple[str, Any], ...]
+
+    @property
+    def key(self) -> KernelKey:
+        idx = self.device.index
+        return KernelKey(device_ordinal=0 if idx is None else idx, params=self.params)

@@ -1,0 +1,188 @@
+"""On-device configuration sweep with recorded choices.
+
+The reference predicts the best tile configuration with per-device XGBoost
+models downloaded from its release page
+(spio/kernels/performance_model_cache.py:102-124, 226-240, 432-479).  Here the
+choice is measured: on the first request for a (kernel, params) pair every
+legal configuration is compiled, timed on the device with HIP events over
+rotating synthetic buffers, and the fastest one is recorded in a JSON file
+keyed by device name and full kernel name.  Later processes read the record
+and compile only the winner.
+
+Environment:
+  SPIO_TUNE=0      never sweep; use the first (heuristically best) configuration
+  SPIO_TUNE=1      sweep on a miss (default)
+  SPIO_TUNE=force  sweep even when a record exists
+  SPIO_TUNE_DB     path of the record file (default: <cache dir>/tune/<device>.json)
+"""
+
+import dataclasses
+import json
+import os
+import threading
+import time
+from typing import Any, Dict, List, Optional
+
+from ..compiler.compiler_pool import compile_kernel_configs
+from ..util.cache_dir import get_cache_dir
+from ..util.logger import logger_enabled
+
+_PACKAGE_RECORDS = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tuned")
+
+# Rotate the timed launches over buffer sets totalling at least this many bytes
+# so that the sweep ranks configurations by their HBM behaviour, not by hits in
+# the 256 MB memory-side cache.
+ROTATION_BYTES = 600 * 1024 * 1024
+MAX_ROTATION_SETS = 8
+
+
+def _mode() -> str:
+    return os.environ.get("SPIO_TUNE", "1").strip().lower()
+
+
+def _device_file_name(device_name: str) -> str:
+    safe = "".join(ch if ch.isalnum() else "_" for ch in device_name.strip().lower())
+    return (safe or "unknown_device") + ".json"
+
+
+def config_to_dict(config) -> Dict[str, Any]:
+    return dataclasses.asdict(config)
+
+
+class Tuner:
+    """Picks (and remembers) the fastest configuration of a kernel."""
+
+    def __init__(self):
+        self._lock = threading.RLock()
+        self._records: Dict[str, Dict[str, Any]] = {}  # device file name -> records
+        self.last_sweep: Optional[List[Dict[str, Any]]] = None
+
+    # -- record storage -------------------------------------------------
+    def _user_path(self, device_name: str) -> str:
+        override = os.environ.get("SPIO_TUNE_DB")
+        if override:
+            return override
+        return os.path.join(get_cache_dir("tune"), _device_file_name(device_name))
+
+    def _load(self, device_name: str) -> Dict[str, Any]:
+        fname = _device_file_name(device_name)
+        recs = self._records.get(fname)
+        if recs is not None:
+            return recs
+        recs = {}
+        for path in (os.path.join(_PACKAGE_RECORDS, fname), self._user_path(device_name)):
+            try:
+                with open(path, "r", encoding="utf-8") as f:
+                    recs.update(json.load(f))
+            except (OSError, ValueError):
+                pass
+        self._records[fname] = recs
+        return recs
+
+    def _store(self, device_name: str, kernel_name: str, record: Dict[str, Any]):
+        recs = self._load(device_name)
+        recs[kernel_name] = record
+        path = self._user_path(device_name)
+        try:
+            on_disk = {}
+            try:
+                with open(path, "r", encoding="utf-8") as f:
+                    on_disk = json.load(f)
+            except (OSError, ValueError):
+                pass
+            on_disk[kernel_name] = record
+            tmp = f"{path}.{os.getpid()}.tmp"
+            with open(tmp, "w", encoding="utf-8") as f:
+                json.dump(on_disk, f, indent=1, sort_keys=True)
+            os.replace(tmp, path)
+        except OSError:
+            pass
+
+    def lookup(self, device_name: str, kernel_name: str) -> Optional[Dict[str, Any]]:
+        """The stored record for a kernel on a device, if any."""
+        with self._lock:
+            return self._load(device_name).get(kernel_name)
+
+    # -- selection ------------------------------------------------------
+    def best_kernel(self, kernel_factory, params, ordinal, device_attr, **kernel_kwargs):
+        """A compiled, loaded kernel using the best known configuration."""
+        from .kernel_cache import compile_and_load_kernel  # circular at import time
+
+        with self._lock:
+            configs = list(kernel_factory.configs(params, device_attr, **kernel_kwargs))
+            if not configs:
+                raise ValueError(f"no kernel configuration supports {params}")
+            name = kernel_factory.get_full_kernel_name(params, **kernel_kwargs)
+            mode = _mode()
+            record = None if mode == "force" else self.lookup(device_attr.name, name)
+            if record is not None:
+                try:
+                    config = kernel_factory.config_cls(**record["config"])
+                except TypeError:
+                    config = None
+                if config in configs:
+                    return compile_and_load_kernel(
+                        kernel_factory, params, config, ordinal, device_attr, **kernel_kwargs
+                    )
+            if mode in ("0", "false", "off", "no") or len(configs) == 1:
+                return compile_and_load_kernel(
+                    kernel_factory, params, configs[0], ordinal, device_attr, **kernel_kwargs
+                )
+            return self.sweep(kernel_factory, params, ordinal, device_attr, configs, **kernel_kwargs)
+
+    def sweep(self, kernel_factory, params, ordinal, device_attr, configs=None, warmup=2,
+              iters=8, **kernel_kwargs):  # fmt: skip
+        """Time every configuration; record and return the fastest kernel (loaded)."""
+        import torch  # pylint: disable=import-outside-toplevel
+
+        if configs is None:
+            configs = list(kernel_factory.configs(params, device_attr, **kernel_kwargs))
+        name = kernel_factory.get_full_kernel_name(params, **kernel_kwargs)
+        t0 = time.perf_counter()
+        kernels = compile_kernel_configs(
+            kernel_factory, params, configs=configs, device_attr=device_attr, **kernel_kwargs
+        )
+        device = torch.device("cuda", ordinal)
+        first = kernel_factory.make_test_args(params, device, **kernel_kwargs)
+        set_bytes = sum(a.numel() * a.element_size() for a in first if hasattr(a, "numel"))
+        nsets = max(1, min(MAX_ROTATION_SETS, -(-ROTATION_BYTES // max(set_bytes, 1))))
+        arg_sets = [first] + [
+            kernel_factory.make_test_args(params, device, **kernel_kwargs) for _ in range(nsets - 1)
+        ]
+        results = []
+        best = None
+        for kernel in kernels:
+            try:
+                kernel.load(device_ordinal=ordinal)
+                ms = kernel.time(arg_sets, warmup=warmup, iters=iters)
+            except ValueError as e:
+                results.append({"config": config_to_dict(kernel.config), "error": str(e)[:200]})
+                kernel.unload()
+                continue
+            results.append({"config": config_to_dict(kernel.config), "us": ms * 1e3})
+            if best is None or ms < best[0]:
+                if best is not None:
+                    best[1].unload()
+                best = (ms, kernel)
+            else:
+                kernel.unload()
+        del arg_sets, first
+        if best is None:
+            raise ValueError(f"every configuration of {name} failed: {results}")
+        record = {
+            "config": config_to_dict(best[1].config),
+            "us": best[0] * 1e3,
+            "candidates": len(configs),
+            "sweep": sorted((r for r in results if "us" in r), key=lambda r: r["us"])[:8],
+        }
+        self._store(device_attr.name, name, record)
+        self.last_sweep = results
+        if logger_enabled:
+            print(
+                f"spio: tuned {name}: {best[1].config} {best[0] * 1e3:.1f} us "
+                f"({len(configs)} configs, {time.perf_counter() - t0:.1f} s)"
+            )
+        return best[1]
+
+
+tuner = Tuner()

@@ -1,0 +1,78 @@
+"""GPU parity of the fprop / dgrad / wgrad kernels against the CPU oracle.
+
+Mirrors the kernel-level tests of the reference (tests/test_conv2d_gw8.py:
+110-201): sanity shapes, the regression shapes, and seeded samples of the full
+shape list, each over several tile configurations, outputs pre-filled with a
+sentinel.
+"""
+
+import pytest
+
+from helpers import run_grad_kernel_test, run_kernel_test, sample_params
+from spio_amd.kernels import (
+    Conv2dGw8Config,
+    Conv2dGw8Params,
+    conv2d_gw8_kernel_factory,
+    conv2d_gw8_wgrad_kernel_factory,
+)
+
+pytestmark = pytest.mark.gpu
+
+SANITY = [
+    Conv2dGw8Params(n=4, c=64, h=16, w=32, padding=1, r=3, s=3, has_bias=True),
+    Conv2dGw8Params(n=4, c=48, h=32, w=32, padding=1, r=3, s=3, has_bias=False),
+    Conv2dGw8Params(n=1, c=64, h=8, w=16, padding=1, r=3, s=3, has_bias=False),
+    Conv2dGw8Params(n=4, c=128, h=32, w=32, padding=(2, 0), r=4, s=1, has_bias=True),
+    Conv2dGw8Params(n=1, c=128, h=64, w=64, padding=7, has_bias=False),
+    Conv2dGw8Params(n=6, c=128, h=6, w=5, has_bias=True),
+    Conv2dGw8Params(n=3, c=24, h=20, w=19, padding=0, has_bias=False),
+    Conv2dGw8Params(n=2, c=40, h=9, w=9, r=5, s=5, padding=2, has_bias=True),
+    Conv2dGw8Params(n=2, c=32, h=14, w=14, r=7, s=7, padding=3, has_bias=False),
+    Conv2dGw8Params(n=5, c=8, h=7, w=7, r=2, s=5, padding=(1, 2), has_bias=True),
+]
+
+
+@pytest.mark.parametrize("params", SANITY, ids=lambda p: p.encode())
+def test_fprop_sanity(params):
+    run_kernel_test(conv2d_gw8_kernel_factory, params)
+
+
+@pytest.mark.parametrize("params", SANITY, ids=lambda p: p.encode())
+def test_dgrad_sanity(params):
+    run_grad_kernel_test(conv2d_gw8_kernel_factory, params, igrad=True)
+
+
+@pytest.mark.parametrize("params", SANITY, ids=lambda p: p.encode())
+def test_wgrad_sanity(params):
+    run_grad_kernel_test(conv2d_gw8_wgrad_kernel_factory, params)
+
+
+def test_fprop_explicit_configs():
+    """Explicit tile configurations, like the reference's regression cases
+    (tests/test_conv2d_gw8.py:117-142): a group count that does not divide the
+    channel blocks evenly and a one-image tile."""
+    params = Conv2dGw8Params(n=4, c=48, h=32, w=32, padding=1)
+    run_kernel_test(conv2d_gw8_kernel_factory, params,
+                    configs=[Conv2dGw8Config(groups=4, block_p=8, block_n=2, split=1),
+                             Conv2dGw8Config(groups=6, block_p=7, block_n=1, split=2)])  # fmt: skip
+    params = Conv2dGw8Params(n=1, c=64, h=8, w=16, padding=1)
+    run_kernel_test(conv2d_gw8_kernel_factory, params,
+                    configs=[Conv2dGw8Config(groups=8, block_p=8, block_n=1)])  # fmt: skip
+
+
+@pytest.mark.slow
+@pytest.mark.parametrize("params", sample_params(seed=1), ids=lambda p: p.encode())
+def test_fprop_sampled(params):
+    run_kernel_test(conv2d_gw8_kernel_factory, params)
+
+
+@pytest.mark.slow
+@pytest.mark.parametrize("params", sample_params(seed=2), ids=lambda p: p.encode())
+def test_dgrad_sampled(params):
+    run_grad_kernel_test(conv2d_gw8_kernel_factory, params, igrad=True)
+
+
+@pytest.mark.slow
+@pytest.mark.parametrize("params", sample_params(seed=3), ids=lambda p: p.encode())
+def test_wgrad_sampled(params):
+    run_grad_kernel_test(conv2d_gw8_wgrad_kernel_factory, params)
