@@ -1,0 +1,165 @@
+"""GPU parity of the operator, its autograd, autocast, layer and registration.
+
+Mirrors the function / layer / opcheck tests of the reference
+(tests/test_conv2d_gw8.py:176-236; procedures spio/src_tests/run_test.py:128-246):
+the op is called on fp32 arguments under torch.autocast so the AutocastCUDA
+implementation runs, gradients come from torch.autograd.grad, and everything is
+compared with the fp32 CPU oracle.
+"""
+
+import pytest
+import torch
+from torch import nn
+
+from helpers import sample_params, to_gpu
+from oracle import conv2d_gw8_oracle as oracle
+from spio_amd.functional import conv2d_gw8
+from spio_amd.kernels import Conv2dGw8Params, Conv2dStats
+from spio_amd.layers import Conv2dGw8
+
+pytestmark = pytest.mark.gpu
+
+FUNCTION_SHAPES = [
+    Conv2dGw8Params(n=4, c=128, h=32, w=32, padding=(2, 0), r=4, s=1, has_bias=True),
+    Conv2dGw8Params(n=4, c=64, h=16, w=32, padding=1, r=3, s=3, has_bias=True),
+    Conv2dGw8Params(n=3, c=40, h=9, w=9, padding=2, r=5, s=5, has_bias=False),
+    Conv2dGw8Params(n=1, c=128, h=64, w=64, padding=7, has_bias=False),
+]
+
+
+def _call(params, x, w, b):
+    return conv2d_gw8(x, w, b, stride=1, padding_y=params.padding_h, padding_x=params.padding_w,
+                      groups=params.groups)  # fmt: skip
+
+
+def _depths(params):
+    return Conv2dStats(params, output_names=["output", "grad_input", "grad_weight", "grad_bias"]).accumulation_depths
+
+
+def run_function_test(params, seed=0):
+    x, w, b, _dy = oracle.make_args(params.n, params.c, params.h, params.w, params.r, params.s,
+                                    params.padding_h, params.padding_w, params.has_bias, seed)  # fmt: skip
+    expected = oracle.fprop_torch(x, w, b, params.padding_h, params.padding_w)
+    # fp32 arguments under autocast: exercises the AutocastCUDA implementation.
+    xg, wg, bg = to_gpu(x).float(), to_gpu(w).float(), to_gpu(b)
+    with torch.autocast(device_type="cuda", dtype=torch.float16):
+        y = _call(params, xg, wg, bg)
+    assert y.dtype == torch.float32  # cast back to the input dtype
+    oracle.check_close(y, expected, acc_depth=_depths(params)[0], what=f"function {params.encode()}")
+    # fp16 arguments without autocast
+    y16 = _call(params, to_gpu(x), to_gpu(w), bg)
+    assert y16.dtype == torch.float16 and y16.is_contiguous(memory_format=torch.channels_last)
+    oracle.check_close(y16, expected, acc_depth=_depths(params)[0], what=f"function fp16 {params.encode()}")
+
+
+def run_grad_function_test(params, seed=0):
+    x, w, b, dy = oracle.make_args(params.n, params.c, params.h, params.w, params.r, params.s,
+                                   params.padding_h, params.padding_w, params.has_bias, seed)  # fmt: skip
+    dx_e, dw_e, db_e = oracle.grads_torch(x, w, b, dy, params.padding_h, params.padding_w)
+    xg = to_gpu(x).float().requires_grad_(True)
+    wg = to_gpu(w).float().requires_grad_(True)
+    bg = to_gpu(b).requires_grad_(True) if b is not None else None
+    with torch.autocast(device_type="cuda", dtype=torch.float16):
+        y = _call(params, xg, wg, bg)
+    leaves = [xg, wg] + ([bg] if bg is not None else [])
+    grads = torch.autograd.grad(y, leaves, to_gpu(dy).float())
+    d = _depths(params)
+    oracle.check_close(grads[0], dx_e, acc_depth=d[1], what=f"grad_input {params.encode()}")
+    oracle.check_close(grads[1], dw_e, acc_depth=d[2], what=f"grad_weight {params.encode()}")
+    assert grads[1].dtype == torch.float32
+    if bg is not None:
+        oracle.check_close(grads[2], db_e, acc_depth=d[3], what=f"grad_bias {params.encode()}")
+
+
+@pytest.mark.parametrize("params", FUNCTION_SHAPES, ids=lambda p: p.encode())
+def test_function(params):
+    run_function_test(params)
+
+
+@pytest.mark.parametrize("params", FUNCTION_SHAPES, ids=lambda p: p.encode())
+def test_function_grad(params):
+    run_grad_function_test(params)
+
+
+@pytest.mark.slow
+@pytest.mark.parametrize("params", sample_params(seed=4, count=6), ids=lambda p: p.encode())
+def test_function_sampled(params):
+    run_function_test(params, seed=1)
+    run_grad_function_test(params, seed=1)
+
+
+def test_backward_op_skips_what_is_not_needed():
+    p = Conv2dGw8Params(n=2, c=16, h=8, w=8, has_bias=True)
+    x, w, b, dy = oracle.make_args(p.n, p.c, p.h, p.w, 3, 3, 1, 1, True, 0)
+    args = (to_gpu(x), to_gpu(w), to_gpu(b), to_gpu(dy), 1, 1)
+    dx, dw, db = torch.ops.spio.conv2d_gw8_backward(*args, False, True, False)
+    assert dx is None and db is None and dw.dtype == torch.float32 and dw.shape == w.shape
+    dx, dw, db = torch.ops.spio.conv2d_gw8_backward(*args, True, False, True)
+    assert dw is None and dx.dtype == torch.float16 and db.dtype == torch.float32
+    # only the input requires grad
+    xg = to_gpu(x).requires_grad_(True)
+    y = _call(p, xg, to_gpu(w), to_gpu(b))
+    (gx,) = torch.autograd.grad(y, (xg,), to_gpu(dy))
+    oracle.check_close(gx, oracle.grads_torch(x, w, b, dy, 1, 1)[0], acc_depth=72, what="dx only")
+
+
+def test_wgrad_accumulates_into_its_output():
+    """The weight-gradient kernel adds to grad_weight: two launches give exactly twice one
+    launch's contribution (up to the order of fp32 atomics)."""
+    from spio_amd.kernels import conv2d_gw8_wgrad_kernel_factory
+
+    p = Conv2dGw8Params(n=2, c=16, h=8, w=8)
+    x, w, _b, dy = oracle.make_args(p.n, p.c, p.h, p.w, 3, 3, 1, 1, False, 0)
+    kernel = conv2d_gw8_wgrad_kernel_factory.get_kernel(p, torch.device("cuda", 0))
+    dw = torch.zeros(p.weight_shape, device="cuda").contiguous(memory_format=torch.channels_last)
+    kernel(dw, to_gpu(x), to_gpu(dy))
+    once = dw.clone()
+    kernel(dw, to_gpu(x), to_gpu(dy))
+    torch.cuda.synchronize()
+    assert torch.allclose(dw, 2 * once, rtol=1e-5, atol=1e-4)
+    oracle.check_close(once, oracle.grads_torch(x, w, None, dy, 1, 1)[1], acc_depth=128, what="wgrad once")
+
+
+def test_non_channels_last_arguments_are_accepted():
+    """NCHW-contiguous inputs and weights are converted, like the reference's to_channels_last."""
+    p = Conv2dGw8Params(n=2, c=16, h=8, w=8)
+    x, w, _b, _dy = oracle.make_args(p.n, p.c, p.h, p.w, 3, 3, 1, 1, False, 0)
+    y = _call(p, x.contiguous().cuda(), w.contiguous().cuda(), None)
+    oracle.check_close(y, oracle.fprop_torch(x, w, None, 1, 1), acc_depth=72, what="nchw args")
+
+
+@pytest.mark.parametrize("torchcompile", [False, True])
+def test_layer(torchcompile):
+    """An nn.Conv2d and the Conv2dGw8 sharing its parameters give the same result."""
+    torch.manual_seed(0)
+    conv = nn.Conv2d(64, 64, 3, padding=1, groups=8).cuda().to(memory_format=torch.channels_last)
+    layer = Conv2dGw8.from_torch_module(conv)
+    run = torch.compile(layer) if torchcompile else layer
+    x = torch.randn(4, 64, 20, 24, device="cuda").contiguous(memory_format=torch.channels_last)
+    with torch.autocast(device_type="cuda", dtype=torch.float16):
+        y = run(x)
+    expected = oracle.fprop_torch(x.half(), conv.weight.half(), conv.bias, 1, 1)
+    oracle.check_close(y, expected, acc_depth=72, what="layer")
+
+
+def test_layer_training_step():
+    """fp32 master weights + autocast: gradients land in fp32 on the parameters."""
+    torch.manual_seed(1)
+    layer = Conv2dGw8(32, 32, 3, padding=1, groups=4).cuda().to(memory_format=torch.channels_last)
+    x = torch.randn(2, 32, 12, 12, device="cuda").contiguous(memory_format=torch.channels_last)
+    with torch.autocast(device_type="cuda", dtype=torch.float16):
+        y = layer(x)
+    dy = torch.randn_like(y)
+    y.backward(dy)
+    assert layer.weight.grad.dtype == torch.float32 and layer.bias.grad.dtype == torch.float32
+    _dx, dw_e, db_e = oracle.grads_torch(x.half(), layer.weight.detach().half(), layer.bias.detach(), dy.half(), 1, 1)
+    oracle.check_close(layer.weight.grad, dw_e, acc_depth=2 * 12 * 12, what="layer dw")
+    oracle.check_close(layer.bias.grad, db_e, acc_depth=2 * 12 * 12, what="layer db")
+
+
+def test_opcheck():
+    p = Conv2dGw8Params(n=4, c=64, h=16, w=32, padding=1, has_bias=True)
+    x, w, b, _ = oracle.make_args(p.n, p.c, p.h, p.w, 3, 3, 1, 1, True, 0)
+    args = (to_gpu(x).requires_grad_(True), to_gpu(w).requires_grad_(True), to_gpu(b).requires_grad_(True))
+    kwargs = dict(stride=1, padding_y=1, padding_x=1, dilation=1, groups=p.groups)
+    torch.library.opcheck(conv2d_gw8, args, kwargs)

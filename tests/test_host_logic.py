@@ -1,0 +1,133 @@
+"""Host-side kernel infrastructure without a GPU: configuration spaces, launch
+geometry, JIT specialisation of every kernel family, caches and the tuner's
+record store.  CPU only."""
+
+import json
+
+import pytest
+
+from helpers import reference_test_params
+from spio_amd.hip import DeviceAttributes
+from spio_amd.kernels import (
+    Conv2dGw8Config,
+    Conv2dGw8Params,
+    KernelCache,
+    KernelKey,
+    KernelParamsLogger,
+    LaunchParams,
+    conv2d_gw8_kernel_factory,
+    conv2d_gw8_wgrad_kernel_factory,
+    kernel_params_logging_is_enabled,
+)
+from spio_amd.kernels.conv2d_gw8_kernel import MAX_LDS_BYTES, mfma_geometry
+from spio_amd.kernels.tuner import Tuner
+
+ATTR = DeviceAttributes()
+
+
+def test_launch_params_normalisation():
+    lp = LaunchParams(grid=7, block=(64, 2))
+    assert lp.grid == (7, 1, 1) and lp.block == (64, 2, 1)
+    with pytest.raises(AssertionError):
+        LaunchParams(grid=0, block=64)
+    with pytest.raises(ValueError):
+        LaunchParams(grid=(1, 1, 1, 1), block=64)
+
+
+@pytest.mark.parametrize("igrad", [False, True])
+def test_every_shape_has_legal_configs(igrad):
+    """Every shape of the reference's test list gets configurations whose derived
+    geometry respects the device limits, and the direct kernel closes the list."""
+    for params in reference_test_params(False):
+        configs = conv2d_gw8_kernel_factory.configs(params, ATTR, igrad=igrad)
+        assert configs and configs[-1].variant == "direct"
+        assert len(set(configs)) == len(configs)
+        for cfg in configs[:-1]:
+            g = mfma_geometry(params, cfg, igrad)
+            assert g["THREADS"] <= 1024 and g["LDS_BYTES"] <= MAX_LDS_BYTES
+            assert g["NUM_BLOCKS"] >= 1 and g["WT"] * 16 >= g["F"] - params.s + 1
+            assert g["GS"] % 16 == 9 and g["GS"] >= 16 * g["WT"] + 4 * g["KB"] - 1
+            spec = conv2d_gw8_kernel_factory.get_kernel_spec(params, cfg, ATTR, igrad=igrad)
+            assert spec.launch_params.grid[0] == g["NUM_BLOCKS"]
+            assert spec.launch_params.block[0] == g["THREADS"]
+
+
+def test_kernel_names_follow_the_reference_convention():
+    p = Conv2dGw8Params(n=4, c=64, h=16, w=32, has_bias=True)
+    f = conv2d_gw8_kernel_factory
+    assert f.get_full_kernel_name(p) == "spio_conv2d_gw8_fprop__4n_64c_16h_32w_1py_1px_3r_3s_b"
+    assert f.get_full_kernel_name(p, igrad=True).startswith("spio_conv2d_gw8_dgrad__")
+    assert conv2d_gw8_wgrad_kernel_factory.get_full_kernel_name(p).startswith("spio_conv2d_gw8_wgrad__")
+    assert f.get_kernel_cache() is f.get_kernel_cache()
+    assert f.get_kernel_cache() is not f.get_kernel_cache(igrad=True)
+
+
+@pytest.mark.parametrize(
+    "params",
+    [
+        Conv2dGw8Params(n=4, c=64, h=16, w=32, has_bias=True),
+        Conv2dGw8Params(n=3, c=24, h=20, w=19, padding=(2, 0), r=4, s=1),
+        Conv2dGw8Params(n=2, c=32, h=14, w=14, padding=3, r=7, s=7),
+    ],
+    ids=lambda p: p.encode(),
+)
+def test_jit_specialisation_of_every_family(params):
+    """hipRTC compiles first/last configuration of each family for gfx950 (no GPU needed)."""
+    for factory, kw in ((conv2d_gw8_kernel_factory, {}), (conv2d_gw8_kernel_factory, {"igrad": True}),
+                        (conv2d_gw8_wgrad_kernel_factory, {})):  # fmt: skip
+        configs = list(factory.configs(params, ATTR, **kw))
+        for cfg in {configs[0], configs[-1]}:
+            kernel = factory.make_kernel(params, cfg, ATTR, **kw)
+            kernel.compile()
+            assert kernel.code[:4] == b"\x7fELF"
+            assert kernel.kernel_name.encode() in kernel.code
+            with pytest.raises(ValueError):
+                kernel.launch()  # not loaded
+
+
+def test_illegal_config_is_rejected():
+    p = Conv2dGw8Params(n=1, c=64, h=8, w=16)
+    with pytest.raises(AssertionError):
+        conv2d_gw8_kernel_factory.get_kernel_spec(p, Conv2dGw8Config(groups=16, split=4), ATTR)
+    with pytest.raises(ValueError):
+        conv2d_gw8_kernel_factory.get_kernel_spec(p, Conv2dGw8Config(variant="nope"), ATTR)
+
+
+def test_overlay_cache_semantics():
+    """A non-empty overlay must contain the key (reference: kernel_cache.py:62-68)."""
+    import torch
+
+    cache = KernelCache()
+    p = Conv2dGw8Params(n=1, c=8, h=4, w=4)
+    sentinel = object()
+    cache.update_overlay({KernelKey(device_ordinal=0, params=p): sentinel})
+    dev = torch.device("cuda", 0)
+    assert cache.get(conv2d_gw8_kernel_factory, p, dev) is sentinel
+    with pytest.raises(ValueError, match="overlay"):
+        cache.get(conv2d_gw8_kernel_factory, Conv2dGw8Params(n=2, c=8, h=4, w=4), dev)
+    cache.clear_overlay()
+
+
+def test_params_logger_records_requests():
+    import torch
+
+    cache = KernelCache()
+    p = Conv2dGw8Params(n=1, c=8, h=4, w=4)
+    cache.update_overlay({KernelKey(device_ordinal=0, params=p): object()})
+    assert not kernel_params_logging_is_enabled()
+    with KernelParamsLogger() as logger:
+        assert kernel_params_logging_is_enabled()
+        cache.get(conv2d_gw8_kernel_factory, p, torch.device("cuda", 0), igrad=True)
+    assert not kernel_params_logging_is_enabled()
+    (rec,) = logger.get_logged_params()
+    assert rec.params == p and rec.kernel_kwargs == (("igrad", True),)
+    assert rec.key == KernelKey(device_ordinal=0, params=p)
+
+
+def test_tuner_record_store(tmp_path, monkeypatch):
+    monkeypatch.setenv("SPIO_TUNE_DB", str(tmp_path / "db.json"))
+    t = Tuner()
+    assert t.lookup("Some GPU", "k__x") is None
+    t._store("Some GPU", "k__x", {"config": {"groups": 8}, "us": 12.5})
+    assert Tuner().lookup("Some GPU", "k__x")["us"] == 12.5
+    assert json.load(open(tmp_path / "db.json"))["k__x"]["config"] == {"groups": 8}
