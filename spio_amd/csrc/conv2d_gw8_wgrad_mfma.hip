@@ -1,0 +1,295 @@
+// Row-streaming MFMA kernel for the conv2d_gw8 weight gradient (gfx950).
+//
+// Contract (reference kernel: spio/src/conv2d_gw8_wgrad.cu:10-226):
+//   dw[k,r,s,c] += sum_{n,p,q} x[n,p+r-py,q+s-px,8g+c] * dy[n,p,q,k]      g = k / 8
+// fp16 operands, fp32 accumulation, fp32 result added into `grad_weight`
+// ([K][R][S][8] floats) with atomics, so the caller zeroes it first
+// (spio/functional/conv2d_gw8_function.py:124-130).
+//
+// Design
+//   * A workgroup owns SPIO_BH rows of dy (output rows) of SPIO_NB images side
+//     by side, for SPIO_GB channel groups, and repeats that for SPIO_ITERS
+//     image blocks before it publishes its sums.  Per step it stages one row
+//     of x and one row of dy in LDS ([group][flattened pixel][8 ch], zero
+//     halo materialised once, as in the forward kernel).
+//   * One wave owns one group.  The contraction runs over pixels, so both MFMA
+//     operands need "8 pixels of one channel" per lane while memory holds
+//     "8 channels of one pixel"; the transposing LDS read of gfx950
+//     (ds_read_b64_tr_b16) delivers exactly that from the pixel-major rows.
+//   * v_mfma_f32_16x16x32_f16 per 32-pixel chunk:
+//         A (16 x 32) = dy:  rows m = 8*j + k    (two dy rows j of an aligned row pair, 8 k)
+//         B (32 x 16) = x:   cols n = 8*sj + c   (two column taps sj, 8 c)
+//     so one MFMA yields dw for 2 filter rows x 2 filter columns.  For the x
+//     row of step t and the dy row pair (2i, 2i+1) the filter rows are
+//     r = delta - j with delta = t - 2i in [0, R]; there is one accumulator per
+//     (delta, column-tap pair).  Entries with r or s out of range are never read.
+//   * At the end dw[k,r,s,c] = acc[delta=r] (lanes with j=0) + acc[delta=r+1]
+//     (lanes with j=1); the halves are combined in registers and added to
+//     global memory with one fp32 atomic per element.
+#include "spio_conv_common.h"
+
+using namespace spio;
+
+#ifndef SPIO_NB
+#define SPIO_NB 1
+#endif
+#ifndef SPIO_ITERS
+#define SPIO_ITERS 1
+#endif
+
+namespace {
+
+constexpr int GB = SPIO_GB;        // groups (waves) per workgroup
+constexpr int BH = SPIO_BH;        // dy rows per workgroup
+constexpr int NB = SPIO_NB;        // images side by side
+constexpr int ITERS = SPIO_ITERS;  // image blocks per workgroup
+constexpr int THREADS = 64 * GB;
+
+constexpr int S2 = 2 * ((kS + 1) / 2);
+constexpr int NBLK = S2 / 2;   // column-tap pairs
+constexpr int ND = kR + 1;     // values of delta
+constexpr int WPI = kQ + kS - 1;  // padded width of one image (= W + 2*px)
+constexpr int F = NB * WPI;
+constexpr int KSPAN = (NB - 1) * WPI + kQ;  // flattened pixels that carry dy
+constexpr int KC = (KSPAN + 31) / 32;       // 32-pixel chunks
+constexpr int FPX = 32 * KC + S2 - 1;
+constexpr int GSX = FPX + ((9 - FPX % 16) + 16) % 16;  // x group stride (pixels), = 9 mod 16
+constexpr int FPD = 32 * KC;
+constexpr int GSD = FPD + ((9 - FPD % 16) + 16) % 16;  // dy group stride
+constexpr int NRX = 2;                                 // x ring rows
+constexpr int NRD = 2 * ((kR + 2) / 2);                // dy ring rows: even, >= R+1
+constexpr int XROW_UNITS = GB * GSX;
+constexpr int DROW_UNITS = GB * GSD;
+constexpr int X_CELLS = F * GB;
+constexpr int LPTX = (X_CELLS + THREADS - 1) / THREADS;
+constexpr int D_CELLS = NB * kQ * GB;
+constexpr int LPTD = (D_CELLS + THREADS - 1) / THREADS;
+constexpr int GBLKS = (kGroups + GB - 1) / GB;
+constexpr int PBLKS = (kP + BH - 1) / BH;
+constexpr int NBLKS = (kN + NB * ITERS - 1) / (NB * ITERS);
+constexpr int NUM_BLOCKS = GBLKS * PBLKS * NBLKS;
+constexpr int STEPS = BH + kR - 1;
+
+static_assert((NRX * XROW_UNITS + NRD * DROW_UNITS) * 16 <= 160 * 1024, "LDS overflow");
+static_assert(NRD % 2 == 0 && NRD >= kR + 1, "dy ring too small");
+
+SPIO_DEVICE spio_half8 read_tr_pair(const unsigned char* lo, const unsigned char* hi) {
+    typedef spio_short4 __attribute__((address_space(3))) * lds_ptr;
+    union {
+        spio_short4 s[2];
+        spio_half8 h;
+    } v;
+    v.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)lo);
+    v.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)hi);
+    return v.h;
+}
+
+}  // namespace
+
+extern "C" __global__ void SPIO_LAUNCH_BOUNDS(THREADS)
+SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__ x,
+                 const spio_uint4* __restrict__ dy) {
+    __shared__ spio_uint4 xring[NRX * XROW_UNITS];
+    __shared__ spio_uint4 dring[NRD * DROW_UNITS];
+
+    const int tid = thread_id();
+    const int lane = tid & 63;
+    const int wg = tid >> 6;  // group within the workgroup
+
+    int b = block_id();
+    if (NUM_BLOCKS % 8 == 0) b = (b & 7) * (NUM_BLOCKS / 8) + (b >> 3);
+    const int pb = b % PBLKS;
+    const int cb = (b / PBLKS) % GBLKS;
+    const int nbk = b / (PBLKS * GBLKS);
+    const int p0 = pb * BH;
+    const int bh_eff = imin(BH, kP - p0);  // dy rows that exist in this block
+    const int gglob = cb * GB + wg;
+    const bool wave_active = gglob < kGroups;
+
+    // zero both rings once: halo, gap and slack cells are never written again
+    for (int i = tid; i < NRX * XROW_UNITS; i += THREADS) xring[i] = spio_uint4{0u, 0u, 0u, 0u};
+    for (int i = tid; i < NRD * DROW_UNITS; i += THREADS) dring[i] = spio_uint4{0u, 0u, 0u, 0u};
+
+    // lane roles inside the transposing reads: block kb = lane/16 covers pixels 8*kb..8*kb+7,
+    // source lane sigma = lane%16 = 4*jr + t supplies pixel jr (+4 for the second read) of
+    // unit t/2 (dy row j or column tap sj) and channel half t%2.
+    const int kb = lane >> 4;
+    const int jr = (lane & 15) >> 2;
+    const int tt = lane & 3;
+    const int sel = tt >> 1;  // j for A, sj for B
+    const int xfrag_off = ((wg * GSX + 8 * kb + jr + sel) * 16) + (tt & 1) * 8;   // bytes in an x row
+    const int dfrag_off = ((wg * GSD + 8 * kb + jr) * 16) + (tt & 1) * 8;         // bytes in a dy row
+
+    spio_float4 acc[ND][NBLK];
+#pragma unroll
+    for (int d = 0; d < ND; ++d)
+#pragma unroll
+        for (int nb = 0; nb < NBLK; ++nb) acc[d][nb] = spio_float4{0.f, 0.f, 0.f, 0.f};
+
+    const long long xrow_units = (long long)kW * kGroups;
+    const long long drow_units = (long long)kQ * kGroups;
+
+    for (int it = 0; it < ITERS; ++it) {
+        const int n0 = (nbk * ITERS + it) * NB;
+        if (n0 >= kN) break;
+
+        // ---- loop-invariant addressing for this image block ----
+        int x_off[LPTX], x_lds[LPTX];
+#pragma unroll
+        for (int l = 0; l < LPTX; ++l) {
+            const int cell = tid + THREADS * l;
+            x_off[l] = -1;
+            x_lds[l] = -1;
+            if (cell < X_CELLS) {
+                const int g = cell % GB;
+                const int f = cell / GB;
+                const int img = f / WPI;
+                const int col = f % WPI - kPadX;
+                x_lds[l] = g * GSX + f;
+                if (col >= 0 && col < kW && n0 + img < kN && cb * GB + g < kGroups)
+                    x_off[l] = ((n0 + img) * kH * kW + col) * kGroups + cb * GB + g;
+            }
+        }
+        int d_off[LPTD], d_lds[LPTD];
+#pragma unroll
+        for (int l = 0; l < LPTD; ++l) {
+            const int cell = tid + THREADS * l;
+            d_off[l] = -1;
+            d_lds[l] = -1;
+            if (cell < D_CELLS) {
+                const int g = cell % GB;
+                const int q = (cell / GB) % kQ;
+                const int img = cell / (GB * kQ);
+                d_lds[l] = g * GSD + img * WPI + q;
+                if (n0 + img < kN && cb * GB + g < kGroups)
+                    d_off[l] = ((n0 + img) * kP * kQ + q) * kGroups + cb * GB + g;
+            }
+        }
+
+        // ---- prologue: rows 0 and 1 into registers, row 0 into LDS ----
+        spio_uint4 xpre[2][LPTX], dpre[2][LPTD];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int h = p0 + t - kPadY;
+            const bool x_ok = t < STEPS && h >= 0 && h < kH;
+#pragma unroll
+            for (int l = 0; l < LPTX; ++l) {
+                xpre[t][l] = spio_uint4{0u, 0u, 0u, 0u};
+                if (x_ok && x_off[l] >= 0) xpre[t][l] = x[x_off[l] + h * xrow_units];
+            }
+            const bool d_ok = t < bh_eff;
+#pragma unroll
+            for (int l = 0; l < LPTD; ++l) {
+                dpre[t][l] = spio_uint4{0u, 0u, 0u, 0u};
+                if (d_ok && d_off[l] >= 0) dpre[t][l] = dy[d_off[l] + (p0 + t) * drow_units];
+            }
+        }
+        block_sync();  // rings zeroed / previous image block finished
+#pragma unroll
+        for (int l = 0; l < LPTX; ++l)
+            if (x_lds[l] >= 0) xring[x_lds[l]] = xpre[0][l];
+#pragma unroll
+        for (int l = 0; l < LPTD; ++l)
+            if (d_lds[l] >= 0) dring[d_lds[l]] = dpre[0][l];
+        block_sync();
+
+        for (int tb = 0; tb < STEPS; tb += 2) {
+#pragma unroll
+            for (int uu = 0; uu < 2; ++uu) {
+                const int t = tb + uu;
+                if (t >= STEPS) break;
+
+                // 1. prefetch rows t+2
+                {
+                    const int t2 = t + 2;
+                    const int h = p0 + t2 - kPadY;
+                    const bool x_ok = t2 < STEPS && h >= 0 && h < kH;
+#pragma unroll
+                    for (int l = 0; l < LPTX; ++l) {
+                        spio_uint4 v = spio_uint4{0u, 0u, 0u, 0u};
+                        if (x_ok && x_off[l] >= 0) v = x[x_off[l] + h * xrow_units];
+                        xpre[uu][l] = v;
+                    }
+                    const bool d_ok = t2 < bh_eff;
+#pragma unroll
+                    for (int l = 0; l < LPTD; ++l) {
+                        spio_uint4 v = spio_uint4{0u, 0u, 0u, 0u};
+                        if (d_ok && d_off[l] >= 0) v = dy[d_off[l] + (p0 + t2) * drow_units];
+                        dpre[uu][l] = v;
+                    }
+                }
+
+                // 2. x row t against the dy row pairs it overlaps
+                const int hcur = p0 + t - kPadY;
+                if (wave_active && hcur >= 0 && hcur < kH) {
+                    const unsigned char* xrow =
+                        reinterpret_cast<const unsigned char*>(xring + uu * XROW_UNITS) + xfrag_off;
+#pragma unroll
+                    for (int ch = 0; ch < KC; ++ch) {
+                        spio_half8 bfrag[NBLK];
+#pragma unroll
+                        for (int nb = 0; nb < NBLK; ++nb) {
+                            const unsigned char* pb0 = xrow + (32 * ch + 2 * nb) * 16;
+                            bfrag[nb] = read_tr_pair(pb0, pb0 + 4 * 16);
+                        }
+#pragma unroll
+                        for (int d = uu; d < ND; d += 2) {
+                            // delta = d has the parity of t: pair index i = (t - d) / 2
+                            const int i2 = t - d;  // first row of the pair, relative to p0
+                            if (i2 >= 0 && i2 < bh_eff) {
+                                const int slot = (i2 + sel) % NRD;
+                                const unsigned char* pa0 =
+                                    reinterpret_cast<const unsigned char*>(dring + slot * DROW_UNITS) +
+                                    dfrag_off + (32 * ch) * 16;
+                                const spio_half8 afrag = read_tr_pair(pa0, pa0 + 4 * 16);
+#pragma unroll
+                                for (int nb = 0; nb < NBLK; ++nb)
+                                    acc[d][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                        afrag, bfrag[nb], acc[d][nb], 0, 0, 0);
+                            }
+                        }
+                    }
+                }
+
+                // 3. rows t+1 into LDS
+                if (t + 1 < STEPS) {
+                    const int hn = p0 + t + 1 - kPadY;
+                    if (hn >= 0 && hn < kH) {
+#pragma unroll
+                        for (int l = 0; l < LPTX; ++l)
+                            if (x_lds[l] >= 0) xring[((uu + 1) & 1) * XROW_UNITS + x_lds[l]] = xpre[(uu + 1) & 1][l];
+                    }
+                    const int dslot = (t + 1) % NRD;
+#pragma unroll
+                    for (int l = 0; l < LPTD; ++l)
+                        if (d_lds[l] >= 0) dring[dslot * DROW_UNITS + d_lds[l]] = dpre[(uu + 1) & 1][l];
+                }
+                block_sync();
+            }
+        }
+    }
+
+    // ---- publish: dw[k,r,s,c] = acc[r] (j = 0 lanes) + acc[r+1] (j = 1 lanes) ----
+    if (wave_active) {
+        const int j = lane >> 5;
+        const int k4 = 4 * ((lane >> 4) & 1);
+        const int sj = (lane & 15) >> 3;
+        const int c = lane & 7;
+#pragma unroll
+        for (int d = 0; d < ND; ++d) {
+            const int r = d - j;
+#pragma unroll
+            for (int nb = 0; nb < NBLK; ++nb) {
+                const int s = 2 * nb + sj;
+                if (r >= 0 && r < kR && s < kS) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int k = 8 * gglob + k4 + e;
+                        atomic_add_f32(grad_weight + (((long long)k * kR + r) * kS + s) * 8 + c,
+                                       acc[d][nb][e]);
+                    }
+                }
+            }
+        }
+    }
+}

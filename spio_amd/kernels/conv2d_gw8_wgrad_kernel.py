@@ -6,7 +6,7 @@ its partial sums into a pre-zeroed fp32 tensor laid out [K][R][S][8]
 """
 
 from dataclasses import dataclass
-from typing import List
+from typing import Dict, List
 
 import torch
 
@@ -19,6 +19,13 @@ from .kernel_factory import KernelFactory
 from .launch_params import LaunchParams
 
 DIRECT_SOURCE = "conv2d_gw8_direct.hip"
+MFMA_SOURCE = "conv2d_gw8_wgrad_mfma.hip"
+
+MAX_WAVES = 16
+MAX_LDS_BYTES = 96 * 1024
+MAX_LOADS_PER_THREAD = 8
+MAX_ACCUMULATORS = 32
+MAX_CONFIGS = 28
 
 
 @dataclass(frozen=True)
@@ -26,29 +33,94 @@ class Conv2dGw8WgradConfig:
     """Tile configuration of the weight-gradient kernel.
 
     Attributes:
-        groups: channel groups per workgroup.
-        block_h: output rows per workgroup pass.
-        block_n: images accumulated by one workgroup before its atomics.
-        chunks: (direct variant) pixel chunks per group.
-        variant: "mfma" or "direct".
+        groups: channel groups (waves) per workgroup.
+        block_h: rows of grad_output per workgroup.
+        block_n: images whose rows are laid side by side in one staged row.
+        block_n_iters: image blocks a workgroup accumulates before its atomics.
+        chunks: (direct variant only) pixel chunks per group.
+        variant: "mfma" (row-streaming MFMA kernel) or "direct" (any shape).
     """
 
     groups: int = 8
-    block_h: int = 8
+    block_h: int = 14
     block_n: int = 1
-    chunks: int = 64
-    variant: str = "direct"
+    block_n_iters: int = 1
+    chunks: int = 0
+    variant: str = "mfma"
+
+
+def wgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig) -> Dict[str, int]:
+    """Host mirror of the compile-time constants of conv2d_gw8_wgrad_mfma.hip."""
+    r, s = params.r, params.s
+    gb, bh, nb, iters = config.groups, config.block_h, config.block_n, config.block_n_iters
+    s2 = 2 * ((s + 1) // 2)
+    wpi = params.q + s - 1
+    f = nb * wpi
+    kspan = (nb - 1) * wpi + params.q
+    kc = divup(kspan, 32)
+    fpx = 32 * kc + s2 - 1
+    gsx = fpx + ((9 - fpx % 16) + 16) % 16
+    fpd = 32 * kc
+    gsd = fpd + ((9 - fpd % 16) + 16) % 16
+    nrd = 2 * ((r + 2) // 2)
+    threads = 64 * gb
+    g = dict(
+        NBLK=s2 // 2, ND=r + 1, WPI=wpi, F=f, KC=kc, GSX=gsx, GSD=gsd, NRD=nrd, THREADS=threads,
+        LDS_BYTES=(2 * gb * gsx + nrd * gb * gsd) * 16,
+        LPTX=divup(f * gb, threads), LPTD=divup(nb * params.q * gb, threads),
+        GBLKS=divup(params.groups, gb), PBLKS=divup(params.p, bh),
+        NBLKS=divup(params.n, nb * iters), STEPS=bh + r - 1,
+        PIXEL_EFF=kspan and (nb * params.q) / (32.0 * kc),
+    )  # fmt: skip
+    g["NUM_BLOCKS"] = g["GBLKS"] * g["PBLKS"] * g["NBLKS"]
+    return g
+
+
+def _mfma_config_is_legal(params, config) -> bool:
+    g = wgrad_geometry(params, config)
+    return (
+        config.groups <= MAX_WAVES
+        and config.block_h <= params.p
+        and config.block_n * config.block_n_iters <= max(params.n, 1)
+        and g["LDS_BYTES"] <= MAX_LDS_BYTES
+        and g["LPTX"] <= MAX_LOADS_PER_THREAD
+        and g["ND"] * g["NBLK"] <= MAX_ACCUMULATORS
+    )
+
+
+def _mfma_score(params, config, num_cus) -> float:
+    g = wgrad_geometry(params, config)
+    halo_rows = (config.block_h + params.r - 1) / config.block_h
+    group_eff = params.groups / (g["GBLKS"] * config.groups)
+    per_cu = max(1, min(160 * 1024 // g["LDS_BYTES"], 2048 // g["THREADS"], 8))
+    slots = num_cus * per_cu
+    quant = divup(g["NUM_BLOCKS"], slots) * slots / g["NUM_BLOCKS"]
+    # every workgroup ends with R*S*64 atomics per wave: amortise them over its pixels
+    pixels = config.block_h * config.block_n * config.block_n_iters * params.q
+    atomics = 1.0 + 4.0 * params.r * params.s * 64 / (pixels * 16.0)
+    return halo_rows ** 0.5 * quant * atomics / (g["PIXEL_EFF"] * group_eff)
 
 
 def _get_configs(params: Conv2dGw8Params, device_attr=None) -> List[Conv2dGw8WgradConfig]:
+    """Legal configurations, most promising first; direct-kernel configurations close the list."""
     num_cus = getattr(device_attr, "multiprocessor_count", 256) or 256
+    G = params.groups
+    group_choices = sorted({g for g in (4, 8, 16, G) if g <= min(G, MAX_WAVES)}) or [min(G, MAX_WAVES)]
+    row_choices = sorted({bh for bh in (4, 7, 8, 14, 16, 28, 32, 56, params.p) if bh <= params.p})
+    found = []
+    for gb in group_choices:
+        for nb in (1, 2, 4, 8):
+            for iters in (1, 2, 4, 8):
+                for bh in row_choices:
+                    cfg = Conv2dGw8WgradConfig(groups=gb, block_h=bh, block_n=nb, block_n_iters=iters)
+                    if _mfma_config_is_legal(params, cfg):
+                        found.append((_mfma_score(params, cfg, num_cus), cfg))
+    found.sort(key=lambda sc: sc[0])
+    configs = [cfg for _, cfg in found[:MAX_CONFIGS]]
     total_pix = params.n * params.p * params.q
-    configs = []
-    for mult in (4, 2, 8):
-        chunks = max(1, min(divup(mult * num_cus, params.groups), divup(total_pix, 64)))
-        cfg = Conv2dGw8WgradConfig(groups=1, block_h=1, block_n=1, chunks=chunks, variant="direct")
-        if cfg not in configs:
-            configs.append(cfg)
+    chunks = max(1, min(divup(8 * num_cus, params.groups), divup(total_pix, 64)))
+    configs.append(Conv2dGw8WgradConfig(groups=1, block_h=1, block_n=1, block_n_iters=1,
+                                        chunks=chunks, variant="direct"))  # fmt: skip
     return configs
 
 
@@ -61,7 +133,13 @@ def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig, _dev
         return KernelSpec(
             defines, LaunchParams(grid=params.groups * config.chunks, block=threads), DIRECT_SOURCE
         )
-    raise ValueError(f"unknown kernel variant {config.variant!r}")
+    if config.variant != "mfma":
+        raise ValueError(f"unknown kernel variant {config.variant!r}")
+    assert _mfma_config_is_legal(params, config), f"illegal configuration {config} for {params}"
+    g = wgrad_geometry(params, config)
+    defines.update(SPIO_GB=config.groups, SPIO_BH=config.block_h, SPIO_NB=config.block_n,
+                   SPIO_ITERS=config.block_n_iters)  # fmt: skip
+    return KernelSpec(defines, LaunchParams(grid=g["NUM_BLOCKS"], block=g["THREADS"]), MFMA_SOURCE, notes=g)
 
 
 def _make_test_args(params: Conv2dGw8Params, device):
