@@ -115,6 +115,24 @@ int spio_hip_launch_timed(void* function,
                           void*** param_sets, int num_sets, int num_params,
                           int warmup, int iters, float* elapsed_ms);
 
+/* One launch of a multi-kernel sequence (same fields as spio_hip_launch). */
+typedef struct spio_hip_launch_desc {
+    void* function;
+    unsigned grid[3];
+    unsigned block[3];
+    unsigned dynamic_lds_bytes;
+    int num_params;
+    void** params;
+} spio_hip_launch_desc_t;
+
+/* Like spio_hip_launch_timed for operators made of several kernels run back
+ * to back (the two-stage weight gradient).  `descs` holds num_sets * stages
+ * descriptors; iteration i launches the `stages` descriptors of set
+ * i % num_sets in order.  No counterpart in the reference, whose operators
+ * are single kernels. */
+int spio_hip_launch_sequence_timed(const spio_hip_launch_desc_t* descs, int stages, int num_sets,
+                                   void* stream, int warmup, int iters, float* elapsed_ms);
+
 /* Asynchronous fill of a device buffer with zero bytes on `stream`; used for
  * the pre-zeroed weight-gradient contract
  * (spio/functional/conv2d_gw8_function.py:124-127) by callers without torch. */

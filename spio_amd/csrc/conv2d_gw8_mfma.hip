@@ -101,6 +101,18 @@ static_assert(NR * RING_ROW_UNITS * 16 + 2 * OUT_ROW_BYTES <= 160 * 1024, "LDS o
 
 constexpr int pmod(int a, int m) { return ((a % m) + m) % m; }
 
+// Source rows shared with the neighbouring row blocks (the first and last R-1
+// steps) can be served from L2 when the neighbour runs on the same XCD;
+// SPIO_HALO_CACHED = 1 loads those with the default policy and only the
+// interior rows with the non-temporal hint.
+#ifndef SPIO_HALO_CACHED
+#define SPIO_HALO_CACHED 0
+#endif
+SPIO_DEVICE spio_uint4 load_row(const spio_uint4* p, int step) {
+    if (SPIO_HALO_CACHED && (step < kR - 1 || step >= BP)) return *p;
+    return load_stream(p);
+}
+
 }  // namespace
 
 extern "C" __global__ void SPIO_LAUNCH_BOUNDS(THREADS)
@@ -232,7 +244,7 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
 #pragma unroll
         for (int l = 0; l < LPT; ++l) {
             pre[t][l] = spio_uint4{0u, 0u, 0u, 0u};
-            if (row_ok && in_off[l] >= 0) pre[t][l] = src[in_off[l] + h * row_units];
+            if (row_ok && in_off[l] >= 0) pre[t][l] = load_row(src + in_off[l] + h * row_units, t);
         }
     }
     block_sync();  // ring zeroed
@@ -266,7 +278,7 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
 #pragma unroll
                 for (int l = 0; l < LPT; ++l) {
                     spio_uint4 v = spio_uint4{0u, 0u, 0u, 0u};
-                    if (row_ok && in_off[l] >= 0) v = src[in_off[l] + h * row_units];
+                    if (row_ok && in_off[l] >= 0) v = load_row(src + in_off[l] + h * row_units, tt);
                     pre[pbuf][l] = v;
                 }
             }
@@ -345,7 +357,7 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
                         if (out_off[s] >= 0) {
                             const spio_uint4 v = *reinterpret_cast<const spio_uint4*>(
                                 ostage + obuf * OUT_ROW_BYTES + out_lds[s]);
-                            dst[out_off[s] + p * dst_row_units] = v;
+                            store_stream(v, dst + out_off[s] + p * dst_row_units);
                         }
                     }
                 }

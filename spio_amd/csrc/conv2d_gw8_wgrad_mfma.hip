@@ -24,8 +24,13 @@
 //     r = delta - j with delta = t - 2i in [0, R]; there is one accumulator per
 //     (delta, column-tap pair).  Entries with r or s out of range are never read.
 //   * At the end dw[k,r,s,c] = acc[delta=r] (lanes with j=0) + acc[delta=r+1]
-//     (lanes with j=1); the halves are combined in registers and added to
-//     global memory with one fp32 atomic per element.
+//     (lanes with j=1); the halves are combined through LDS.  fp32 atomics are
+//     the scarce resource (the device retires roughly 128 per clock in total,
+//     and every workgroup owes R*S*64 of them per group), so there are two
+//     ways to publish: SPIO_PARTIALS=0 adds straight into grad_weight with
+//     atomics; SPIO_PARTIALS=1 stores each workgroup's sums into its own
+//     partial image of a workspace with plain stores, and the small
+//     <name>_reduce kernel below folds the partial images into grad_weight.
 #include "spio_conv_common.h"
 
 using namespace spio;
@@ -36,6 +41,12 @@ using namespace spio;
 #ifndef SPIO_ITERS
 #define SPIO_ITERS 1
 #endif
+#ifndef SPIO_PF
+#define SPIO_PF 2
+#endif
+#ifndef SPIO_PARTIALS
+#define SPIO_PARTIALS 0
+#endif
 
 namespace {
 
@@ -44,6 +55,7 @@ constexpr int BH = SPIO_BH;        // dy rows per workgroup
 constexpr int NB = SPIO_NB;        // images side by side
 constexpr int ITERS = SPIO_ITERS;  // image blocks per workgroup
 constexpr int THREADS = 64 * GB;
+constexpr int PF = SPIO_PF;  // prefetch distance in rows (even)
 
 constexpr int S2 = 2 * ((kS + 1) / 2);
 constexpr int NBLK = S2 / 2;   // column-tap pairs
@@ -59,7 +71,9 @@ constexpr int GSD = FPD + ((9 - FPD % 16) + 16) % 16;  // dy group stride
 constexpr int NRX = 2;                                 // x ring rows
 constexpr int NRD = 2 * ((kR + 2) / 2);                // dy ring rows: even, >= R+1
 constexpr int XROW_UNITS = GB * GSX;
-constexpr int DROW_UNITS = GB * GSD;
+// dy ring rows are 64 bytes apart modulo the 256-byte bank period, so the two rows of a
+// pair that one transposing read touches fall into different banks.
+constexpr int DROW_UNITS = GB * GSD + ((4 - (GB * GSD) % 16) + 16) % 16;
 constexpr int X_CELLS = F * GB;
 constexpr int LPTX = (X_CELLS + THREADS - 1) / THREADS;
 constexpr int D_CELLS = NB * kQ * GB;
@@ -72,6 +86,7 @@ constexpr int STEPS = BH + kR - 1;
 
 static_assert((NRX * XROW_UNITS + NRD * DROW_UNITS) * 16 <= 160 * 1024, "LDS overflow");
 static_assert(NRD % 2 == 0 && NRD >= kR + 1, "dy ring too small");
+static_assert(PF >= 2 && PF % 2 == 0, "prefetch distance must be even");
 
 SPIO_DEVICE spio_half8 read_tr_pair(const unsigned char* lo, const unsigned char* hi) {
     typedef spio_short4 __attribute__((address_space(3))) * lds_ptr;
@@ -166,22 +181,22 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
             }
         }
 
-        // ---- prologue: rows 0 and 1 into registers, row 0 into LDS ----
-        spio_uint4 xpre[2][LPTX], dpre[2][LPTD];
+        // ---- prologue: rows 0..PF-1 into registers, row 0 into LDS ----
+        spio_uint4 xpre[PF][LPTX], dpre[PF][LPTD];
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
+        for (int t = 0; t < PF; ++t) {
             const int h = p0 + t - kPadY;
             const bool x_ok = t < STEPS && h >= 0 && h < kH;
 #pragma unroll
             for (int l = 0; l < LPTX; ++l) {
                 xpre[t][l] = spio_uint4{0u, 0u, 0u, 0u};
-                if (x_ok && x_off[l] >= 0) xpre[t][l] = x[x_off[l] + h * xrow_units];
+                if (x_ok && x_off[l] >= 0) xpre[t][l] = load_stream(x + x_off[l] + h * xrow_units);
             }
             const bool d_ok = t < bh_eff;
 #pragma unroll
             for (int l = 0; l < LPTD; ++l) {
                 dpre[t][l] = spio_uint4{0u, 0u, 0u, 0u};
-                if (d_ok && d_off[l] >= 0) dpre[t][l] = dy[d_off[l] + (p0 + t) * drow_units];
+                if (d_ok && d_off[l] >= 0) dpre[t][l] = load_stream(dy + d_off[l] + (p0 + t) * drow_units);
             }
         }
         block_sync();  // rings zeroed / previous image block finished
@@ -193,29 +208,30 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
             if (d_lds[l] >= 0) dring[d_lds[l]] = dpre[0][l];
         block_sync();
 
-        for (int tb = 0; tb < STEPS; tb += 2) {
+        for (int tb = 0; tb < STEPS; tb += PF) {
 #pragma unroll
-            for (int uu = 0; uu < 2; ++uu) {
-                const int t = tb + uu;
+            for (int uf = 0; uf < PF; ++uf) {
+                const int t = tb + uf;
                 if (t >= STEPS) break;
+                const int uu = uf & 1;  // parity of t: x ring row and the parity of delta
 
-                // 1. prefetch rows t+2
+                // 1. prefetch rows t+PF (their register buffer held row t, now in LDS)
                 {
-                    const int t2 = t + 2;
+                    const int t2 = t + PF;
                     const int h = p0 + t2 - kPadY;
                     const bool x_ok = t2 < STEPS && h >= 0 && h < kH;
 #pragma unroll
                     for (int l = 0; l < LPTX; ++l) {
                         spio_uint4 v = spio_uint4{0u, 0u, 0u, 0u};
-                        if (x_ok && x_off[l] >= 0) v = x[x_off[l] + h * xrow_units];
-                        xpre[uu][l] = v;
+                        if (x_ok && x_off[l] >= 0) v = load_stream(x + x_off[l] + h * xrow_units);
+                        xpre[uf][l] = v;
                     }
                     const bool d_ok = t2 < bh_eff;
 #pragma unroll
                     for (int l = 0; l < LPTD; ++l) {
                         spio_uint4 v = spio_uint4{0u, 0u, 0u, 0u};
-                        if (d_ok && d_off[l] >= 0) v = dy[d_off[l] + (p0 + t2) * drow_units];
-                        dpre[uu][l] = v;
+                        if (d_ok && d_off[l] >= 0) v = load_stream(dy + d_off[l] + (p0 + t2) * drow_units);
+                        dpre[uf][l] = v;
                     }
                 }
 
@@ -257,39 +273,86 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
                     if (hn >= 0 && hn < kH) {
 #pragma unroll
                         for (int l = 0; l < LPTX; ++l)
-                            if (x_lds[l] >= 0) xring[((uu + 1) & 1) * XROW_UNITS + x_lds[l]] = xpre[(uu + 1) & 1][l];
+                            if (x_lds[l] >= 0) xring[((uu + 1) & 1) * XROW_UNITS + x_lds[l]] = xpre[(uf + 1) % PF][l];
                     }
                     const int dslot = (t + 1) % NRD;
 #pragma unroll
                     for (int l = 0; l < LPTD; ++l)
-                        if (d_lds[l] >= 0) dring[dslot * DROW_UNITS + d_lds[l]] = dpre[(uu + 1) & 1][l];
+                        if (d_lds[l] >= 0) dring[dslot * DROW_UNITS + d_lds[l]] = dpre[(uf + 1) % PF][l];
                 }
                 block_sync();
             }
         }
     }
 
-    // ---- publish: dw[k,r,s,c] = acc[r] (j = 0 lanes) + acc[r+1] (j = 1 lanes) ----
+    // ---- publish ----
+    // dw[k,r,s,c] = acc[delta = r] (lanes 0-31: j = 0) + acc[delta = r+1] (lanes 32-63: j = 1).
+    // The j = 1 halves travel through a 512-byte per-wave LDS scratch (LDS operations of one
+    // wave execute in order, so no barrier is needed inside the wave) and lanes 0-31 publish
+    // complete sums: fp32 atomics into grad_weight, or plain stores into this workgroup's
+    // partial image when a second kernel does the reduction.
+    block_sync();  // every wave is done with the rings; reuse the x ring as scratch
     if (wave_active) {
-        const int j = lane >> 5;
+        float* scratch = reinterpret_cast<float*>(xring) + wg * 128;
         const int k4 = 4 * ((lane >> 4) & 1);
         const int sj = (lane & 15) >> 3;
         const int c = lane & 7;
+#if SPIO_PARTIALS
+        float* out = grad_weight + (long long)(nbk * PBLKS + pb) * ((long long)kC * kR * kS * 8);
+#else
+        float* out = grad_weight;
+#endif
 #pragma unroll
-        for (int d = 0; d < ND; ++d) {
-            const int r = d - j;
+        for (int r = 0; r < kR; ++r) {
 #pragma unroll
             for (int nb = 0; nb < NBLK; ++nb) {
                 const int s = 2 * nb + sj;
-                if (r >= 0 && r < kR && s < kS) {
+                if (lane >= 32) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) scratch[e * 32 + (lane - 32)] = acc[r + 1][nb][e];
+                }
+                if (lane < 32) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const int k = 8 * gglob + k4 + e;
-                        atomic_add_f32(grad_weight + (((long long)k * kR + r) * kS + s) * 8 + c,
-                                       acc[d][nb][e]);
+                        const float total = acc[r][nb][e] + scratch[e * 32 + lane];
+                        if (s < kS) {
+                            float* dst = out + (((long long)(8 * gglob + k4 + e) * kR + r) * kS + s) * 8 + c;
+#if SPIO_PARTIALS
+                            *dst = total;
+#else
+                            atomic_add_f32(dst, total);
+#endif
+                        }
                     }
                 }
             }
         }
     }
 }
+
+#if SPIO_PARTIALS
+// Second stage: grad_weight[e] += sum over partial images.  Thread (column of 4 floats,
+// slice) adds the partial images p = slice, slice + SLICES, ... and publishes with atomics, so
+// the result accumulates onto whatever grad_weight holds, like the single-stage kernel.
+#ifndef SPIO_REDUCE_SLICES
+#define SPIO_REDUCE_SLICES 1
+#endif
+#define SPIO_CONCAT2(a, b) a##b
+#define SPIO_CONCAT(a, b) SPIO_CONCAT2(a, b)
+extern "C" __global__ void SPIO_LAUNCH_BOUNDS(256)
+SPIO_CONCAT(SPIO_KERNEL_NAME, _reduce)(float* __restrict__ grad_weight, const spio_float4* __restrict__ partials) {
+    constexpr int COLS = kC * kR * kS * 2;  // float4 columns of one image
+    constexpr int NPART = NBLKS * PBLKS;
+    constexpr int SLICES = SPIO_REDUCE_SLICES;
+    const int idx = block_id() * 256 + thread_id();
+    if (idx >= COLS * SLICES) return;
+    const int col = idx % COLS;
+    const int slice = idx / COLS;
+    spio_float4 sum = spio_float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+    for (int p = slice; p < NPART; p += SLICES) sum += partials[(long long)p * COLS + col];
+    float* dst = grad_weight + 4 * (long long)col;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) atomic_add_f32(dst + e, sum[e]);
+}
+#endif

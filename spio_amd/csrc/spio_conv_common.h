@@ -63,6 +63,27 @@ SPIO_DEVICE void block_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 }
 
+// Streaming accesses: activations are touched once per kernel, so they are
+// loaded and stored with the non-temporal hint (measured on MI355X: a plain
+// 16-byte-per-lane copy gains about 10% from it).
+#ifndef SPIO_NT
+#define SPIO_NT 1
+#endif
+SPIO_DEVICE spio_uint4 load_stream(const spio_uint4* p) {
+#if SPIO_NT
+    return __builtin_nontemporal_load(p);
+#else
+    return *p;
+#endif
+}
+SPIO_DEVICE void store_stream(spio_uint4 v, spio_uint4* p) {
+#if SPIO_NT
+    __builtin_nontemporal_store(v, p);
+#else
+    *p = v;
+#endif
+}
+
 // Device-scope fp32 add without a return value.
 SPIO_DEVICE void atomic_add_f32(float* address, float value) {
     __hip_atomic_fetch_add(address, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -377,6 +377,51 @@ int spio_hip_launch_timed(void* function, unsigned grid_x, unsigned grid_y, unsi
     return SPIO_HIP_OK;
 }
 
+int spio_hip_launch_sequence_timed(const spio_hip_launch_desc_t* descs, int stages, int num_sets,
+                                   void* stream, int warmup, int iters, float* elapsed_ms) {
+    REQUIRE_READY();
+    if (!descs || stages < 1 || num_sets < 1 || warmup < 0 || iters < 1 || !elapsed_ms)
+        return fail(SPIO_HIP_ERR_ARGUMENT, "spio_hip_launch_sequence_timed: bad argument");
+    for (int i = 0; i < stages * num_sets; ++i) {
+        const spio_hip_launch_desc_t& d = descs[i];
+        int rc = check_launch_args(d.function, d.grid[0], d.grid[1], d.grid[2], d.block[0],
+                                   d.block[1], d.block[2], d.num_params);
+        if (rc) return rc;
+        if (d.num_params > 0 && !d.params)
+            return fail(SPIO_HIP_ERR_ARGUMENT, "launch sequence: null params");
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipEvent_t start = nullptr, stop = nullptr;
+    HIP_TRY(hipEventCreate(&start));
+    hipError_t e = g_api.hipEventCreate(&stop);
+    if (e != hipSuccess) {
+        (void)g_api.hipEventDestroy(start);
+        return hip_fail(e, "hipEventCreate");
+    }
+    auto run = [&](int set) {
+        hipError_t err = hipSuccess;
+        for (int st = 0; st < stages && err == hipSuccess; ++st) {
+            const spio_hip_launch_desc_t& d = descs[set * stages + st];
+            err = g_api.hipModuleLaunchKernel(static_cast<hipFunction_t>(d.function), d.grid[0],
+                                              d.grid[1], d.grid[2], d.block[0], d.block[1],
+                                              d.block[2], d.dynamic_lds_bytes, s, d.params, nullptr);
+        }
+        return err;
+    };
+    int set = 0;
+    e = hipSuccess;
+    for (int i = 0; i < warmup && e == hipSuccess; ++i, set = (set + 1) % num_sets) e = run(set);
+    if (e == hipSuccess) e = g_api.hipEventRecord(start, s);
+    for (int i = 0; i < iters && e == hipSuccess; ++i, set = (set + 1) % num_sets) e = run(set);
+    if (e == hipSuccess) e = g_api.hipEventRecord(stop, s);
+    if (e == hipSuccess) e = g_api.hipEventSynchronize(stop);
+    if (e == hipSuccess) e = g_api.hipEventElapsedTime(elapsed_ms, start, stop);
+    (void)g_api.hipEventDestroy(start);
+    (void)g_api.hipEventDestroy(stop);
+    if (e != hipSuccess) return hip_fail(e, "timed launch sequence");
+    return SPIO_HIP_OK;
+}
+
 int spio_hip_memset_zero_async(void* device_ptr, size_t bytes, void* stream) {
     REQUIRE_READY();
     if (!device_ptr && bytes) return fail(SPIO_HIP_ERR_ARGUMENT, "memset: null pointer");

@@ -22,4 +22,5 @@ from .driver import (
     stream_synchronize,
     set_device,
     memset_zero_async,
+    launch_sequence_timed,
 )

@@ -35,6 +35,17 @@ class _DeviceAttrsStruct(ctypes.Structure):
     ]
 
 
+class _LaunchDesc(ctypes.Structure):
+    _fields_ = [
+        ("function", ctypes.c_void_p),
+        ("grid", ctypes.c_uint * 3),
+        ("block", ctypes.c_uint * 3),
+        ("dynamic_lds_bytes", ctypes.c_uint),
+        ("num_params", ctypes.c_int),
+        ("params", ctypes.POINTER(ctypes.c_void_p)),
+    ]
+
+
 @dataclass(frozen=True)
 class DeviceAttributes:
     """Static properties of one GPU.
@@ -80,6 +91,11 @@ _SIGNATURES = {
         [_vp] + [ctypes.c_uint] * 7
         + [_vp, ctypes.POINTER(ctypes.POINTER(_vp)), ctypes.c_int, ctypes.c_int, ctypes.c_int,
            ctypes.c_int, ctypes.POINTER(ctypes.c_float)],
+        ctypes.c_int,
+    ),
+    "spio_hip_launch_sequence_timed": (
+        [ctypes.POINTER(_LaunchDesc), ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int, ctypes.c_int,
+         ctypes.POINTER(ctypes.c_float)],
         ctypes.c_int,
     ),
     "spio_hip_memset_zero_async": ([_vp, ctypes.c_size_t, _vp], ctypes.c_int),
@@ -317,6 +333,40 @@ class Function:
             )  # fmt: skip
         )
         return ms.value / iters
+
+
+def launch_sequence_timed(launch_sets, stream: int = 0, warmup: int = 3, iters: int = 20) -> float:
+    """Average milliseconds per iteration of a multi-kernel sequence.
+
+    `launch_sets` is a list of argument sets; each set is a list of stages
+    `(function, grid, block, shared_mem_bytes, args)` launched in order.
+    Iterations cycle through the sets.
+    """
+    init()
+    stages = len(launch_sets[0])
+    descs = (_LaunchDesc * (stages * len(launch_sets)))()
+    keep = []
+    i = 0
+    for launch_set in launch_sets:
+        assert len(launch_set) == stages
+        for function, grid, block, lds, args in launch_set:
+            arr, storage = Function.marshal(args)
+            keep.append((arr, storage))
+            d = descs[i]
+            d.function = function.handle
+            d.grid = (ctypes.c_uint * 3)(*grid)
+            d.block = (ctypes.c_uint * 3)(*block)
+            d.dynamic_lds_bytes = int(lds)
+            d.num_params = len(storage)
+            d.params = ctypes.cast(arr, ctypes.POINTER(ctypes.c_void_p))
+            i += 1
+    ms = ctypes.c_float()
+    _check(
+        _lib.spio_hip_launch_sequence_timed(
+            descs, stages, len(launch_sets), stream or None, int(warmup), int(iters), ctypes.byref(ms)
+        )
+    )
+    return ms.value / iters
 
 
 class Module:

@@ -28,6 +28,7 @@ MAX_LDS_BYTES = 64 * 1024
 MAX_LOADS_PER_THREAD = 8
 MAX_ACCUMULATORS = 16
 MAX_CONFIGS = 28
+PREFETCH_CHOICES = (2, 4, 8)
 
 
 @dataclass(frozen=True)
@@ -40,6 +41,9 @@ class Conv2dGw8Config:
         block_n: images whose rows are laid side by side in one staged row.
         split: waves sharing the 16-pixel tiles of one group.
         prefetch: rows of global loads in flight ahead of the computed row.
+        nontemporal: 1 = stream activations with the non-temporal hint.
+        halo_cached: 1 = load rows shared with neighbouring row blocks with the default
+            cache policy so the second reader can hit in L2.
         variant: "mfma" (row-streaming MFMA kernel) or "direct" (one thread per
             output pixel-group; any shape).
     """
@@ -50,6 +54,8 @@ class Conv2dGw8Config:
     split: int = 1
     prefetch: int = 2
     variant: str = "mfma"
+    nontemporal: int = 1
+    halo_cached: int = 0
 
 
 def direction_geometry(params: Conv2dGw8Params, igrad: bool) -> Dict[str, int]:
@@ -98,7 +104,7 @@ def _mfma_config_is_legal(params, config, igrad) -> bool:
         and g["LPT"] <= MAX_LOADS_PER_THREAD
         and g["TPW"] * g["NACC"] <= MAX_ACCUMULATORS
         and config.prefetch >= 2
-        and g["UNROLL"] <= 12
+        and g["UNROLL"] <= 16
     )
 
 
@@ -129,9 +135,10 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None, igrad: bool = False)
         for nb in (1, 2, 4, 8):
             for ts in (1, 2, 4):
                 for bp in row_choices:
-                    cfg = Conv2dGw8Config(groups=gb, block_p=bp, block_n=nb, split=ts)
-                    if _mfma_config_is_legal(params, cfg, igrad):
-                        found.append((_mfma_score(params, cfg, igrad, num_cus), cfg))
+                    for pf in PREFETCH_CHOICES:
+                        cfg = Conv2dGw8Config(groups=gb, block_p=bp, block_n=nb, split=ts, prefetch=pf)
+                        if _mfma_config_is_legal(params, cfg, igrad):
+                            found.append((_mfma_score(params, cfg, igrad, num_cus), cfg))
     found.sort(key=lambda sc: sc[0])
     configs = [cfg for _, cfg in found[:MAX_CONFIGS]]
     configs.append(Conv2dGw8Config(groups=1, block_p=1, block_n=1, split=1, variant="direct"))
@@ -166,6 +173,7 @@ def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8Config, _device_a
     defines.update(
         SPIO_GB=config.groups, SPIO_BP=config.block_p, SPIO_NB=config.block_n,
         SPIO_TS=config.split, SPIO_PF=config.prefetch,
+        SPIO_NT=config.nontemporal, SPIO_HALO_CACHED=config.halo_cached,
     )  # fmt: skip
     return KernelSpec(
         defines, LaunchParams(grid=g["NUM_BLOCKS"], block=g["THREADS"]), MFMA_SOURCE, notes=g

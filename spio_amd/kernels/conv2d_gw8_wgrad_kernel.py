@@ -26,6 +26,7 @@ MAX_LDS_BYTES = 96 * 1024
 MAX_LOADS_PER_THREAD = 8
 MAX_ACCUMULATORS = 32
 MAX_CONFIGS = 28
+REDUCE_TARGET_THREADS = 64 * 1024
 
 
 @dataclass(frozen=True)
@@ -38,6 +39,9 @@ class Conv2dGw8WgradConfig:
         block_n: images whose rows are laid side by side in one staged row.
         block_n_iters: image blocks a workgroup accumulates before its atomics.
         chunks: (direct variant only) pixel chunks per group.
+        prefetch: rows of global loads in flight ahead of the computed row (even).
+        two_stage: 1 = workgroups store partial sums to a workspace and a second kernel
+            reduces them; 0 = workgroups add into grad_weight with fp32 atomics.
         variant: "mfma" (row-streaming MFMA kernel) or "direct" (any shape).
     """
 
@@ -47,6 +51,8 @@ class Conv2dGw8WgradConfig:
     block_n_iters: int = 1
     chunks: int = 0
     variant: str = "mfma"
+    prefetch: int = 2
+    two_stage: int = 0
 
 
 def wgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig) -> Dict[str, int]:
@@ -66,7 +72,7 @@ def wgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig) -> Dic
     threads = 64 * gb
     g = dict(
         NBLK=s2 // 2, ND=r + 1, WPI=wpi, F=f, KC=kc, GSX=gsx, GSD=gsd, NRD=nrd, THREADS=threads,
-        LDS_BYTES=(2 * gb * gsx + nrd * gb * gsd) * 16,
+        LDS_BYTES=(2 * gb * gsx + nrd * (gb * gsd + ((4 - (gb * gsd) % 16) + 16) % 16)) * 16,
         LPTX=divup(f * gb, threads), LPTD=divup(nb * params.q * gb, threads),
         GBLKS=divup(params.groups, gb), PBLKS=divup(params.p, bh),
         NBLKS=divup(params.n, nb * iters), STEPS=bh + r - 1,
@@ -85,6 +91,9 @@ def _mfma_config_is_legal(params, config) -> bool:
         and g["LDS_BYTES"] <= MAX_LDS_BYTES
         and g["LPTX"] <= MAX_LOADS_PER_THREAD
         and g["ND"] * g["NBLK"] <= MAX_ACCUMULATORS
+        and config.prefetch >= 2
+        and config.prefetch % 2 == 0
+        and (g["LPTX"] + g["LPTD"]) * config.prefetch <= 32
     )
 
 
@@ -138,8 +147,17 @@ def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig, _dev
     assert _mfma_config_is_legal(params, config), f"illegal configuration {config} for {params}"
     g = wgrad_geometry(params, config)
     defines.update(SPIO_GB=config.groups, SPIO_BH=config.block_h, SPIO_NB=config.block_n,
-                   SPIO_ITERS=config.block_n_iters)  # fmt: skip
-    return KernelSpec(defines, LaunchParams(grid=g["NUM_BLOCKS"], block=g["THREADS"]), MFMA_SOURCE, notes=g)
+                   SPIO_ITERS=config.block_n_iters, SPIO_PF=config.prefetch)  # fmt: skip
+    spec = KernelSpec(defines, LaunchParams(grid=g["NUM_BLOCKS"], block=g["THREADS"]), MFMA_SOURCE, notes=g)
+    if config.two_stage:
+        num_partials = g["NBLKS"] * g["PBLKS"]
+        cols = params.c * params.r * params.s * 2  # float4 columns of one partial image
+        slices = max(1, min(num_partials, divup(REDUCE_TARGET_THREADS, cols)))
+        defines.update(SPIO_PARTIALS=1, SPIO_REDUCE_SLICES=slices)
+        spec.workspace_bytes = num_partials * cols * 16
+        spec.epilogue_suffix = "_reduce"
+        spec.epilogue_launch_params = LaunchParams(grid=divup(cols * slices, 256), block=256)
+    return spec
 
 
 def _make_test_args(params: Conv2dGw8Params, device):

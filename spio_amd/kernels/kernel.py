@@ -12,6 +12,7 @@ import torch
 
 from ..compiler.compile_kernel import compile_kernel, load_kernel
 from ..compiler import flags
+from ..hip.driver import launch_sequence_timed
 from ..util.memory_format import check_channels_last
 from .launch_params import LaunchParams
 
@@ -32,6 +33,12 @@ class KernelSpec:
     source_file: str
     max_dynamic_lds: Optional[int] = None
     notes: Dict[str, object] = field(default_factory=dict)
+    # Two-stage kernels: the main kernel receives a workspace of `workspace_bytes` in place of
+    # its first argument, then `<kernel name><epilogue_suffix>` runs with (first argument,
+    # workspace) under `epilogue_launch_params`.
+    workspace_bytes: int = 0
+    epilogue_suffix: Optional[str] = None
+    epilogue_launch_params: Optional[LaunchParams] = None
 
 
 class Kernel:
@@ -47,6 +54,7 @@ class Kernel:
         self.code: Optional[bytes] = None
         self.module = None
         self.function = None
+        self.epilogue_function = None
         self.device_ordinal: Optional[int] = None
 
     @property
@@ -72,6 +80,10 @@ class Kernel:
             raise ValueError(f"Kernel {self.kernel_name} has not been compiled")
         self.module, self.function = load_kernel(self.kernel_name, self.code, device_ordinal)
         self.device_ordinal = device_ordinal
+        if self.kernel_spec.epilogue_suffix:
+            self.epilogue_function = self.module.get_function(
+                self.kernel_name + self.kernel_spec.epilogue_suffix
+            )
         if self.kernel_spec.max_dynamic_lds:
             self.function.set_max_dynamic_lds(self.kernel_spec.max_dynamic_lds)
         if clear_code:
@@ -83,6 +95,7 @@ class Kernel:
             self.module.unload()
             self.module = None
         self.function = None
+        self.epilogue_function = None
 
     def _prepare(self, args):
         if self.function is None:
@@ -103,24 +116,46 @@ class Kernel:
         """Asynchronous launch on torch's current stream of the arguments' device."""
         try:
             device, kargs = self._prepare(args)
-            lp = self.kernel_spec.launch_params
+            spec = self.kernel_spec
+            lp = spec.launch_params
             stream = torch.cuda.current_stream(device).cuda_stream
-            self.function.launch(lp.grid, lp.block, kargs, lp.shared_mem_bytes, stream)
+            if self.epilogue_function is None:
+                self.function.launch(lp.grid, lp.block, kargs, lp.shared_mem_bytes, stream)
+            else:
+                workspace = self._workspace(device)
+                self.function.launch(lp.grid, lp.block, [workspace] + kargs[1:], lp.shared_mem_bytes, stream)
+                ep = spec.epilogue_launch_params
+                self.epilogue_function.launch(ep.grid, ep.block, [kargs[0], workspace], ep.shared_mem_bytes, stream)
         except Exception as e:
             raise ValueError(f"Error in kernel {self}") from e
 
+    def _workspace(self, device) -> torch.Tensor:
+        """Scratch for the partial results of a two-stage kernel (from torch's caching allocator)."""
+        return torch.empty(self.kernel_spec.workspace_bytes, dtype=torch.uint8, device=device)
+
     def time(self, arg_sets, warmup: int = 3, iters: int = 20) -> float:
-        """Average milliseconds per launch, HIP events on torch's current stream."""
+        """Average milliseconds per call (all stages), HIP events on torch's current stream."""
         device = None
         prepared = []
         for args in arg_sets:
             device, kargs = self._prepare(args)
             prepared.append(kargs)
-        lp = self.kernel_spec.launch_params
+        spec = self.kernel_spec
+        lp = spec.launch_params
         stream = torch.cuda.current_stream(device).cuda_stream
-        return self.function.launch_timed(
-            lp.grid, lp.block, prepared, lp.shared_mem_bytes, stream, warmup, iters
-        )
+        if self.epilogue_function is None:
+            return self.function.launch_timed(
+                lp.grid, lp.block, prepared, lp.shared_mem_bytes, stream, warmup, iters
+            )
+        ep = spec.epilogue_launch_params
+        sets = []
+        for kargs in prepared:
+            ws = self._workspace(device)
+            sets.append([
+                (self.function, lp.grid, lp.block, lp.shared_mem_bytes, [ws] + kargs[1:]),
+                (self.epilogue_function, ep.grid, ep.block, ep.shared_mem_bytes, [kargs[0], ws]),
+            ])  # fmt: skip
+        return launch_sequence_timed(sets, stream, warmup, iters)
 
     def __call__(self, *args):
         self.launch(*args)
