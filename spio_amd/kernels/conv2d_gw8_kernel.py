@@ -27,8 +27,8 @@ MAX_WAVES = 16
 MAX_LDS_BYTES = 64 * 1024
 MAX_LOADS_PER_THREAD = 8
 MAX_ACCUMULATORS = 16
-MAX_CONFIGS = 28
-PREFETCH_CHOICES = (2, 4, 8)
+MAX_CONFIGS = 32
+PREFETCH_CHOICES = (2, 4, 8, 16)
 
 
 @dataclass(frozen=True)
@@ -105,22 +105,40 @@ def _mfma_config_is_legal(params, config, igrad) -> bool:
         and g["TPW"] * g["NACC"] <= MAX_ACCUMULATORS
         and config.prefetch >= 2
         and g["UNROLL"] <= 16
+        and g["LPT"] * config.prefetch <= 24
     )
 
 
+def _resident_workgroups(lds_bytes: int, threads: int) -> int:
+    """Workgroups of one kernel a CU can hold (LDS and thread limits)."""
+    return max(1, min(160 * 1024 // max(lds_bytes, 1), 2048 // threads, 8))
+
+
 def _mfma_score(params, config, igrad, num_cus: int) -> float:
-    """Rough relative cost used only to order (and cap) the sweep."""
+    """Rough relative cost used only to order (and cap) the sweep; lower is better.
+
+    The kernel is HBM-bound, so the model prices extra traffic (halo rows),
+    idle compute units (grid quantisation), too few bytes in flight (prefetch
+    depth x resident workgroups) and, weakly, wasted MFMA columns.
+    """
     g = mfma_geometry(params, config, igrad)
-    halo_rows = (config.block_p + params.r - 1) / config.block_p
+    halo = (config.block_p + params.r - 1) / config.block_p
+    traffic = 1.0 + 0.5 * (halo - 1.0)
     useful = config.block_n * g["DW"]
     tile_eff = useful / (16.0 * g["WT"])
     group_eff = params.groups / (g["GBLKS"] * config.groups)
-    # Workgroups per CU limited by LDS and by 2048 threads.
-    per_cu = max(1, min(160 * 1024 // g["LDS_BYTES"], 2048 // g["THREADS"], 8))
-    slots = num_cus * per_cu
-    waves_of_blocks = divup(g["NUM_BLOCKS"], slots)
-    quant = waves_of_blocks * slots / g["NUM_BLOCKS"]
-    return halo_rows ** 0.5 * quant / (tile_eff * group_eff)
+    per_cu = _resident_workgroups(g["LDS_BYTES"], g["THREADS"])
+    # compute units idle in the last round of workgroups
+    quant = divup(g["NUM_BLOCKS"], num_cus) * num_cus / g["NUM_BLOCKS"]
+    resident = min(per_cu, max(1, g["NUM_BLOCKS"] // num_cus))
+    row_bytes = g["F"] * config.groups * 16
+    in_flight = resident * min(config.prefetch, g["STEPS"]) * row_bytes
+    starve = 1.0 + 0.6 * max(0.0, (64 * 1024 - in_flight) / (64 * 1024))
+    few_waves = 1.15 if resident * g["THREADS"] < 512 else 1.0
+    big_block = 1.08 if g["THREADS"] > 512 else 1.0
+    # a workgroup that covers only part of a 128-byte line of a pixel shares it with another one
+    split_line = 1.0 if (config.groups * 16) % 128 == 0 or config.groups == params.groups else 1.12
+    return traffic * quant * starve * few_waves * big_block * split_line / (tile_eff ** 0.3 * group_eff)
 
 
 def _get_configs(params: Conv2dGw8Params, device_attr=None, igrad: bool = False) -> List[Conv2dGw8Config]:
@@ -135,7 +153,10 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None, igrad: bool = False)
         for nb in (1, 2, 4, 8):
             for ts in (1, 2, 4):
                 for bp in row_choices:
+                    steps = bp + params.r - 1
                     for pf in PREFETCH_CHOICES:
+                        if pf > 2 and pf > steps:
+                            continue
                         cfg = Conv2dGw8Config(groups=gb, block_p=bp, block_n=nb, split=ts, prefetch=pf)
                         if _mfma_config_is_legal(params, cfg, igrad):
                             found.append((_mfma_score(params, cfg, igrad, num_cus), cfg))

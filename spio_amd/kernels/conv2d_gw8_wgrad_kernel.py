@@ -25,7 +25,7 @@ MAX_WAVES = 16
 MAX_LDS_BYTES = 96 * 1024
 MAX_LOADS_PER_THREAD = 8
 MAX_ACCUMULATORS = 32
-MAX_CONFIGS = 28
+MAX_CONFIGS = 32
 REDUCE_TARGET_THREADS = 64 * 1024
 
 
@@ -98,20 +98,32 @@ def _mfma_config_is_legal(params, config) -> bool:
 
 
 def _mfma_score(params, config, num_cus) -> float:
+    """Rough relative cost used only to order (and cap) the sweep; lower is better."""
     g = wgrad_geometry(params, config)
-    halo_rows = (config.block_h + params.r - 1) / config.block_h
+    halo = (config.block_h + params.r - 1) / config.block_h
+    traffic = 1.0 + 0.5 * (halo - 1.0)
     group_eff = params.groups / (g["GBLKS"] * config.groups)
     per_cu = max(1, min(160 * 1024 // g["LDS_BYTES"], 2048 // g["THREADS"], 8))
-    slots = num_cus * per_cu
-    quant = divup(g["NUM_BLOCKS"], slots) * slots / g["NUM_BLOCKS"]
-    # every workgroup ends with R*S*64 atomics per wave: amortise them over its pixels
-    pixels = config.block_h * config.block_n * config.block_n_iters * params.q
-    atomics = 1.0 + 4.0 * params.r * params.s * 64 / (pixels * 16.0)
-    return halo_rows ** 0.5 * quant * atomics / (g["PIXEL_EFF"] * group_eff)
+    # compute units idle in the last round of workgroups
+    quant = divup(g["NUM_BLOCKS"], num_cus) * num_cus / g["NUM_BLOCKS"]
+    # Publishing costs R*S*64 values per (workgroup, group): atomics retire at roughly 128 per
+    # clock device-wide; partial stores plus the reduction kernel cost bandwidth and a launch.
+    stream_bytes = 4.0 * params.n * params.c * params.h * params.w
+    stream_us = stream_bytes / 5.0e6
+    values = g["NUM_BLOCKS"] * config.groups * params.r * params.s * 64.0
+    if config.two_stage:
+        publish_us = 4.5 + 2.0 * 4.0 * values / 5.0e6
+    else:
+        publish_us = values / (128 * 2.1e3)
+    few_waves = 1.15 if min(per_cu, max(1, g["NUM_BLOCKS"] // num_cus)) * g["THREADS"] < 512 else 1.0
+    split_line = 1.0 if (config.groups * 16) % 128 == 0 or config.groups == params.groups else 1.12
+    return (traffic * quant * few_waves * split_line / (g["PIXEL_EFF"] ** 0.3 * group_eff)) * (
+        1.0 + publish_us / stream_us
+    )
 
 
 def _get_configs(params: Conv2dGw8Params, device_attr=None) -> List[Conv2dGw8WgradConfig]:
-    """Legal configurations, most promising first; direct-kernel configurations close the list."""
+    """Legal configurations, most promising first; a direct-kernel configuration closes the list."""
     num_cus = getattr(device_attr, "multiprocessor_count", 256) or 256
     G = params.groups
     group_choices = sorted({g for g in (4, 8, 16, G) if g <= min(G, MAX_WAVES)}) or [min(G, MAX_WAVES)]
@@ -121,9 +133,14 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None) -> List[Conv2dGw8Wgr
         for nb in (1, 2, 4, 8):
             for iters in (1, 2, 4, 8):
                 for bh in row_choices:
-                    cfg = Conv2dGw8WgradConfig(groups=gb, block_h=bh, block_n=nb, block_n_iters=iters)
-                    if _mfma_config_is_legal(params, cfg):
-                        found.append((_mfma_score(params, cfg, num_cus), cfg))
+                    for pf in (2, 4, 8):
+                        if pf > 2 and pf > bh + params.r - 1:
+                            continue
+                        for two_stage in (0, 1):
+                            cfg = Conv2dGw8WgradConfig(groups=gb, block_h=bh, block_n=nb, block_n_iters=iters,
+                                                       prefetch=pf, two_stage=two_stage)  # fmt: skip
+                            if _mfma_config_is_legal(params, cfg):
+                                found.append((_mfma_score(params, cfg, num_cus), cfg))
     found.sort(key=lambda sc: sc[0])
     configs = [cfg for _, cfg in found[:MAX_CONFIGS]]
     total_pix = params.n * params.p * params.q

@@ -5,6 +5,11 @@ import sys
 
 import pytest
 
+# The operator tests check results, not speed: use each kernel family's first (heuristically
+# best) configuration instead of running the on-device sweep for every shape.  The sweep itself
+# is covered by tests/test_tuner_gpu.py.
+os.environ.setdefault("SPIO_TUNE", "0")
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
