@@ -83,6 +83,31 @@ def make_buffers(params, seed, nsets, device):
     return w, sets
 
 
+def copy_yardstick(nbytes, nsets, device, iters):
+    """Rate of a plain 16-byte-per-lane non-temporal copy of `nbytes` in and `nbytes` out."""
+    import torch
+
+    from spio_amd.compiler.compile_kernel import compile_and_load_kernel
+
+    _module, fn = compile_and_load_kernel("spio_stream_copy", "stream_copy.hip", {}, device.index or 0)
+    n = nbytes // 16
+    sets = []
+    for _ in range(nsets):
+        src = torch.randint(0, 2**31 - 1, (n * 4,), dtype=torch.int32, device=device)
+        sets.append((torch.empty_like(src), src, n))
+    stream = torch.cuda.current_stream(device).cuda_stream
+    ms = fn.launch_timed(((n + 255) // 256, 1, 1), (256, 1, 1), sets, 0, stream, 5, iters)
+    del sets
+    return {
+        "kernel": "spio_stream_copy",
+        "us": round(ms * 1e3, 2),
+        "bytes": 2 * n * 16,
+        "GB/s": round(2 * n * 16 / (ms * 1e-3) / 1e9, 1),
+        "note": "plain non-temporal copy of one activation tensor in and one out: the HBM rate "
+                "a read-X/write-X kernel reaches on this device",
+    }
+
+
 def cpu_baseline(params_kwargs, seed, sample_batch):
     """The reference's oracle path on the host cores, on a bounded sample of the workload."""
     import torch
@@ -245,8 +270,16 @@ def main():
         "kernels": kernels,
         "roofline": roofline,
     }
+    del arg_sets
+    del sets
+    torch.cuda.empty_cache()
+    result["copy_yardstick"] = copy_yardstick(
+        2 * params.n * params.c * params.h * params.w, nsets, device, iters
+    )
+    result["roofline"]["frac_of_copy_rate"] = round(
+        kernels[dominant]["GB/s"] / result["copy_yardstick"]["GB/s"], 4
+    )
     if not args.no_cpu_baseline:
-        del sets
         torch.cuda.empty_cache()
         result["cpu_baseline"] = cpu_baseline(pkw, seed, args.cpu_sample_batch)
     print(json.dumps(result))

@@ -10,3 +10,24 @@ Public surface (same names as the reference package `spio`):
 __version__ = "0.1.0"
 
 supported_arch = ("gfx950",)
+
+
+def install_as_spio():
+    """Make `import spio...` resolve to this package (for code written against the reference).
+
+    Registers `spio` and its sub-packages `functional`, `layers`, `kernels`, `transform`,
+    `util`, `compiler` as aliases of the spio_amd modules.  Refuses to shadow a real `spio`.
+    """
+    import importlib
+    import sys
+
+    existing = sys.modules.get("spio")
+    if existing is not None and not getattr(existing, "__file__", "").startswith(__path__[0]):
+        raise RuntimeError("a different 'spio' package is already imported")
+    this = sys.modules[__name__]
+    sys.modules["spio"] = this
+    for name in ("functional", "layers", "kernels", "transform", "util", "compiler"):
+        module = importlib.import_module(f"{__name__}.{name}")
+        sys.modules[f"spio.{name}"] = module
+        setattr(this, name, module)
+    return this

@@ -6,14 +6,14 @@ models downloaded from its release page
 choice is measured: on the first request for a (kernel, params) pair every
 legal configuration is compiled, timed on the device with HIP events over
 rotating synthetic buffers, and the fastest one is recorded in a JSON file
-keyed by device name and full kernel name.  Later processes read the record
+keyed by device model (architecture + CU count) and full kernel name.  Later processes read the record
 and compile only the winner.
 
 Environment:
   SPIO_TUNE=0      never sweep; use the first (heuristically best) configuration
   SPIO_TUNE=1      sweep on a miss (default)
   SPIO_TUNE=force  sweep even when a record exists
-  SPIO_TUNE_DB     path of the record file (default: <cache dir>/tune/<device>.json)
+  SPIO_TUNE_DB     path of the record file (default: <cache dir>/tune/<arch>_<CUs>cu.json)
 """
 
 import dataclasses
@@ -40,9 +40,18 @@ def _mode() -> str:
     return os.environ.get("SPIO_TUNE", "1").strip().lower()
 
 
-def _device_file_name(device_name: str) -> str:
-    safe = "".join(ch if ch.isalnum() else "_" for ch in device_name.strip().lower())
-    return (safe or "unknown_device") + ".json"
+def device_key(device_attr) -> str:
+    """Identifies a device model in record file names: architecture and compute-unit count.
+
+    The marketing name is not used: the runtime reports different strings for the same board
+    depending on what is loaded in the process (a profiler, for one).
+    """
+    arch = "".join(ch if ch.isalnum() else "_" for ch in str(device_attr.arch).strip().lower())
+    return f"{arch or 'unknown'}_{int(device_attr.multiprocessor_count)}cu"
+
+
+def _device_file_name(device_attr) -> str:
+    return device_key(device_attr) + ".json"
 
 
 def config_to_dict(config) -> Dict[str, Any]:
@@ -58,19 +67,19 @@ class Tuner:
         self.last_sweep: Optional[List[Dict[str, Any]]] = None
 
     # -- record storage -------------------------------------------------
-    def _user_path(self, device_name: str) -> str:
+    def _user_path(self, device_attr) -> str:
         override = os.environ.get("SPIO_TUNE_DB")
         if override:
             return override
-        return os.path.join(get_cache_dir("tune"), _device_file_name(device_name))
+        return os.path.join(get_cache_dir("tune"), _device_file_name(device_attr))
 
-    def _load(self, device_name: str) -> Dict[str, Any]:
-        fname = _device_file_name(device_name)
+    def _load(self, device_attr) -> Dict[str, Any]:
+        fname = _device_file_name(device_attr)
         recs = self._records.get(fname)
         if recs is not None:
             return recs
         recs = {}
-        for path in (os.path.join(_PACKAGE_RECORDS, fname), self._user_path(device_name)):
+        for path in (os.path.join(_PACKAGE_RECORDS, fname), self._user_path(device_attr)):
             try:
                 with open(path, "r", encoding="utf-8") as f:
                     recs.update(json.load(f))
@@ -79,10 +88,10 @@ class Tuner:
         self._records[fname] = recs
         return recs
 
-    def _store(self, device_name: str, kernel_name: str, record: Dict[str, Any]):
-        recs = self._load(device_name)
+    def _store(self, device_attr, kernel_name: str, record: Dict[str, Any], path: Optional[str] = None):
+        recs = self._load(device_attr)
         recs[kernel_name] = record
-        path = self._user_path(device_name)
+        path = path or self._user_path(device_attr)
         try:
             on_disk = {}
             try:
@@ -98,10 +107,10 @@ class Tuner:
         except OSError:
             pass
 
-    def lookup(self, device_name: str, kernel_name: str) -> Optional[Dict[str, Any]]:
+    def lookup(self, device_attr, kernel_name: str) -> Optional[Dict[str, Any]]:
         """The stored record for a kernel on a device, if any."""
         with self._lock:
-            return self._load(device_name).get(kernel_name)
+            return self._load(device_attr).get(kernel_name)
 
     # -- selection ------------------------------------------------------
     def best_kernel(self, kernel_factory, params, ordinal, device_attr, **kernel_kwargs):
@@ -114,7 +123,7 @@ class Tuner:
                 raise ValueError(f"no kernel configuration supports {params}")
             name = kernel_factory.get_full_kernel_name(params, **kernel_kwargs)
             mode = _mode()
-            record = None if mode == "force" else self.lookup(device_attr.name, name)
+            record = None if mode == "force" else self.lookup(device_attr, name)
             if record is not None:
                 try:
                     config = kernel_factory.config_cls(**record["config"])
@@ -131,7 +140,7 @@ class Tuner:
             return self.sweep(kernel_factory, params, ordinal, device_attr, configs, **kernel_kwargs)
 
     def sweep(self, kernel_factory, params, ordinal, device_attr, configs=None, warmup=2,
-              iters=8, **kernel_kwargs):  # fmt: skip
+              iters=8, record_path=None, **kernel_kwargs):  # fmt: skip
         """Time every configuration; record and return the fastest kernel (loaded)."""
         import torch  # pylint: disable=import-outside-toplevel
 
@@ -175,7 +184,7 @@ class Tuner:
             "candidates": len(configs),
             "sweep": sorted((r for r in results if "us" in r), key=lambda r: r["us"])[:8],
         }
-        self._store(device_attr.name, name, record)
+        self._store(device_attr, name, record, record_path)
         self.last_sweep = results
         if logger_enabled:
             print(

@@ -20,7 +20,7 @@ from spio_amd.kernels import (
     kernel_params_logging_is_enabled,
 )
 from spio_amd.kernels.conv2d_gw8_kernel import MAX_LDS_BYTES, mfma_geometry
-from spio_amd.kernels.tuner import Tuner
+from spio_amd.kernels.tuner import Tuner, device_key
 
 ATTR = DeviceAttributes()
 
@@ -127,7 +127,8 @@ def test_params_logger_records_requests():
 def test_tuner_record_store(tmp_path, monkeypatch):
     monkeypatch.setenv("SPIO_TUNE_DB", str(tmp_path / "db.json"))
     t = Tuner()
-    assert t.lookup("Some GPU", "k__x") is None
-    t._store("Some GPU", "k__x", {"config": {"groups": 8}, "us": 12.5})
-    assert Tuner().lookup("Some GPU", "k__x")["us"] == 12.5
+    assert t.lookup(ATTR, "k__x") is None
+    t._store(ATTR, "k__x", {"config": {"groups": 8}, "us": 12.5})
+    assert Tuner().lookup(ATTR, "k__x")["us"] == 12.5
+    assert device_key(ATTR) == "gfx950_256cu"
     assert json.load(open(tmp_path / "db.json"))["k__x"]["config"] == {"groups": 8}

@@ -2,6 +2,7 @@
 GPU only."""
 
 import json
+from dataclasses import replace
 
 import pytest
 import torch
@@ -49,8 +50,9 @@ def test_wgrad_sweep_covers_both_publish_modes(tmp_path, monkeypatch):
     attr = get_device_attributes(0)
     params = Conv2dGw8Params(n=8, c=64, h=28, w=28)
     configs = list(conv2d_gw8_wgrad_kernel_factory.configs(params, attr))
-    one = next(c for c in configs if c.variant == "mfma" and not c.two_stage)
-    two = next(c for c in configs if c.variant == "mfma" and c.two_stage)
+    first = next(c for c in configs if c.variant == "mfma")
+    one = replace(first, two_stage=0)
+    two = replace(first, two_stage=1)
     tuner = Tuner()
     kernel = tuner.sweep(conv2d_gw8_wgrad_kernel_factory, params, 0, attr, configs=[one, two, configs[-1]])
     assert len([r for r in tuner.last_sweep if "us" in r]) == 3
