@@ -97,7 +97,10 @@ constexpr int gcd_(int a, int b) { return b == 0 ? a : gcd_(b, a % b); }
 constexpr int UNROLL = NS / gcd_(NS, PF) * PF;  // lcm(NS, PF); even, so also a multiple of NR
 
 static_assert(PF >= 2 && WAVES <= 16 && UNROLL % NR == 0, "bad configuration");
-static_assert(NR * RING_ROW_UNITS * 16 + 2 * OUT_ROW_BYTES <= 160 * 1024, "LDS overflow");
+constexpr int STREAM_UNITS = NR * RING_ROW_UNITS + 2 * OUT_ROW_BYTES / 16;
+constexpr int FILTER_UNITS = kIgrad ? GB * 8 * kR * kS : 0;  // staged filters (data gradient only)
+constexpr int LDS_UNITS = STREAM_UNITS > FILTER_UNITS ? STREAM_UNITS : FILTER_UNITS;
+static_assert(LDS_UNITS * 16 <= 160 * 1024, "LDS overflow");
 
 constexpr int pmod(int a, int m) { return ((a % m) + m) % m; }
 
@@ -118,8 +121,11 @@ SPIO_DEVICE spio_uint4 load_row(const spio_uint4* p, int step) {
 extern "C" __global__ void SPIO_LAUNCH_BOUNDS(THREADS)
 SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ src,
                  const spio_half* __restrict__ weights, const float* __restrict__ bias) {
-    __shared__ spio_uint4 ring[NR * RING_ROW_UNITS];
-    __shared__ __attribute__((aligned(16))) unsigned char ostage[2 * OUT_ROW_BYTES];
+    // One LDS block: the source-row ring, then the two output-stage rows.  The data-gradient
+    // mode first uses the same block to stage the filters of the workgroup's groups.
+    __shared__ spio_uint4 lds[LDS_UNITS];
+    spio_uint4* const ring = lds;
+    unsigned char* const ostage = reinterpret_cast<unsigned char*>(lds + NR * RING_ROW_UNITS);
 
     const int tid = thread_id();
     const int lane = tid & 63;
@@ -181,7 +187,8 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
     // Lane (m = lane%16, kb = lane/16): row slot j = m/8, channel m%8, column tap 4u+kb;
     // the filter row of slot j at distance d is r = (d - j) mod NS (none if r >= R).
     spio_half8 wfrag[NS][KB];
-    {
+    if (!kIgrad) {
+        // A[m = out channel ch][c] = w[8g+ch][r][s][c]: 16 contiguous bytes per lane.
         const int m = lane & 15;
         const int kb = lane >> 4;
         const int j = m >> 3;
@@ -194,22 +201,58 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
                 const int s = 4 * u + kb;
                 Pack16 v;
                 v.u = spio_uint4{0u, 0u, 0u, 0u};
-                if (wave_active && r < kR && s < kS) {
-                    if (!kIgrad) {
-                        // A[m = out channel ch][c] = w[8g+ch][r][s][c]
-                        v.u = *reinterpret_cast<const spio_uint4*>(
-                            weights + (((long long)(8 * gglob + ch) * kR + r) * kS + s) * 8);
-                    } else {
-                        // A[m = dx channel ch][jj] = w[8g+jj][R-1-r][S-1-s][ch]
-#pragma unroll
-                        for (int jj = 0; jj < 8; ++jj)
-                            v.h[jj] = weights[(((long long)(8 * gglob + jj) * kR + (kR - 1 - r)) * kS +
-                                               (kS - 1 - s)) * 8 + ch];
-                    }
-                }
+                if (wave_active && r < kR && s < kS)
+                    v.u = *reinterpret_cast<const spio_uint4*>(
+                        weights + (((long long)(8 * gglob + ch) * kR + r) * kS + s) * 8);
                 wfrag[d][u] = v.h;
             }
         }
+    } else {
+        // A[m = dx channel ch][jj] = w[8g+jj][R-1-r][S-1-s][ch]: the filter transposed within
+        // the group.  The workgroup copies its groups' filters to LDS as they lie in memory
+        // ([jj][r][s][8 ch]) and every wave reads its fragments with the transposing LDS read:
+        // in a 16-lane block source lane 4*jr+t supplies 4 channels (half t%2) of row jj = jr for
+        // the row slot t/2, and result lane i receives rows jj = 0..3 of column i = 8*slot + ch.
+        constexpr int WUNITS = GB * 8 * kR * kS;
+        spio_uint4* wlds = lds;  // ring and output stage are not in use yet
+        for (int i = tid; i < WUNITS; i += THREADS) {
+            const int g = i / (8 * kR * kS);
+            const int rem = i % (8 * kR * kS);
+            spio_uint4 v = spio_uint4{0u, 0u, 0u, 0u};
+            if (cb * GB + g < kGroups)
+                v = reinterpret_cast<const spio_uint4*>(weights)[(long long)(cb * GB + g) * (8 * kR * kS) + rem];
+            wlds[i] = v;
+        }
+        block_sync();
+        const int kb = lane >> 4;
+        const int jr = (lane & 15) >> 2;
+        const int t4 = lane & 3;
+        const int src_slot = t4 >> 1;        // slot whose data this lane fetches
+        const int my_slot = (lane & 15) >> 3;  // slot of the fragment row this lane receives
+        typedef spio_short4 __attribute__((address_space(3))) * lds_ptr;
+#pragma unroll
+        for (int d = 0; d < NS; ++d) {
+#pragma unroll
+            for (int u = 0; u < KB; ++u) {
+                const int s = 4 * u + kb;
+                const int r_src = (d - src_slot + NS) % NS;
+                const int r_mine = (d - my_slot + NS) % NS;
+                // clamp the address of dead taps; their result is discarded below
+                const int rr = r_src < kR ? kR - 1 - r_src : 0;
+                const int ss = s < kS ? kS - 1 - s : 0;
+                const unsigned char* base = reinterpret_cast<const unsigned char*>(wlds) +
+                                            ((((wg * 8 + jr) * kR + rr) * kS + ss) * 16) + (t4 & 1) * 8;
+                union {
+                    spio_short4 q[2];
+                    spio_half8 h;
+                } v;
+                v.q[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)base);
+                v.q[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(base + 4 * kR * kS * 16));
+                if (!(wave_active && r_mine < kR && s < kS)) v.h = spio_half8{0, 0, 0, 0, 0, 0, 0, 0};
+                wfrag[d][u] = v.h;
+            }
+        }
+        block_sync();  // everyone has its fragments before the ring is zero-filled
     }
 
     // Accumulator lane layout: D[m = 4*(lane/16)+i][n = lane%16]: pixel n = lane%16,

@@ -82,6 +82,8 @@ def mfma_geometry(params: Conv2dGw8Params, config: Conv2dGw8Config, igrad: bool)
     threads = 64 * gb * ts
     ostride = gb * 16 + 16
     lds = 2 * gb * gs * 16 + 2 * 16 * wt * ostride
+    if igrad:  # the data gradient stages its groups' filters in the same block first
+        lds = max(lds, gb * 8 * r * s * 16)
     d.update(
         NS=ns, NACC=ns // 2, KB=kb, WPI=wpi, F=f, WT=wt, TPW=divup(wt, ts), GS=gs,
         THREADS=threads, LDS_BYTES=lds, LPT=divup(f * gb, threads),
