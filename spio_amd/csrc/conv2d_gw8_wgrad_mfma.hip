@@ -31,6 +31,10 @@
 //     atomics; SPIO_PARTIALS=1 stores each workgroup's sums into its own
 //     partial image of a workspace with plain stores, and the small
 //     <name>_reduce kernel below folds the partial images into grad_weight.
+//     (Reducing inside the kernel by "the last workgroup of a group to finish"
+//     was measured and rejected: the device-scope release/acquire fences it
+//     needs write back and invalidate the L2 of an XCD and cost more than the
+//     atomics they save.)
 #include "spio_conv_common.h"
 
 using namespace spio;
@@ -47,6 +51,9 @@ using namespace spio;
 #ifndef SPIO_PARTIALS
 #define SPIO_PARTIALS 0
 #endif
+#ifndef SPIO_TS
+#define SPIO_TS 1
+#endif
 
 namespace {
 
@@ -54,7 +61,9 @@ constexpr int GB = SPIO_GB;        // groups (waves) per workgroup
 constexpr int BH = SPIO_BH;        // dy rows per workgroup
 constexpr int NB = SPIO_NB;        // images side by side
 constexpr int ITERS = SPIO_ITERS;  // image blocks per workgroup
-constexpr int THREADS = 64 * GB;
+constexpr int TS = SPIO_TS;        // waves sharing the 32-pixel chunks of one group
+constexpr int WAVES = GB * TS;
+constexpr int THREADS = 64 * WAVES;
 constexpr int PF = SPIO_PF;  // prefetch distance in rows (even)
 
 constexpr int S2 = 2 * ((kS + 1) / 2);
@@ -88,6 +97,7 @@ static_assert((NRX * XROW_UNITS + NRD * DROW_UNITS) * 16 <= 160 * 1024, "LDS ove
 static_assert(NRD % 2 == 0 && NRD >= kR + 1, "dy ring too small");
 static_assert(PF >= 2 && PF % 2 == 0, "prefetch distance must be even");
 
+
 SPIO_DEVICE spio_half8 read_tr_pair(const unsigned char* lo, const unsigned char* hi) {
     typedef spio_short4 __attribute__((address_space(3))) * lds_ptr;
     union {
@@ -104,12 +114,16 @@ SPIO_DEVICE spio_half8 read_tr_pair(const unsigned char* lo, const unsigned char
 extern "C" __global__ void SPIO_LAUNCH_BOUNDS(THREADS)
 SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__ x,
                  const spio_uint4* __restrict__ dy) {
-    __shared__ spio_uint4 xring[NRX * XROW_UNITS];
-    __shared__ spio_uint4 dring[NRD * DROW_UNITS];
+    // One LDS block: the x ring, then the dy ring; reused as reduction scratch at the end.
+    __shared__ spio_uint4 lds[NRX * XROW_UNITS + NRD * DROW_UNITS];
+    spio_uint4* const xring = lds;
+    spio_uint4* const dring = lds + NRX * XROW_UNITS;
 
     const int tid = thread_id();
     const int lane = tid & 63;
-    const int wg = tid >> 6;  // group within the workgroup
+    const int wave = tid >> 6;
+    const int wg = wave % GB;  // group within the workgroup
+    const int ws = wave / GB;  // which share of the 32-pixel chunks this wave multiplies
 
     int b = block_id();
     if (NUM_BLOCKS % 8 == 0) b = (b & 7) * (NUM_BLOCKS / 8) + (b >> 3);
@@ -241,7 +255,9 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
                     const unsigned char* xrow =
                         reinterpret_cast<const unsigned char*>(xring + uu * XROW_UNITS) + xfrag_off;
 #pragma unroll
-                    for (int ch = 0; ch < KC; ++ch) {
+                    for (int ci = 0; ci < (KC + TS - 1) / TS; ++ci) {
+                        const int ch = ws + TS * ci;
+                        if (TS > 1 && ch >= KC) break;
                         spio_half8 bfrag[NBLK];
 #pragma unroll
                         for (int nb = 0; nb < NBLK; ++nb) {
@@ -288,12 +304,16 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
     // ---- publish ----
     // dw[k,r,s,c] = acc[delta = r] (lanes 0-31: j = 0) + acc[delta = r+1] (lanes 32-63: j = 1).
     // The j = 1 halves travel through a 512-byte per-wave LDS scratch (LDS operations of one
-    // wave execute in order, so no barrier is needed inside the wave) and lanes 0-31 publish
-    // complete sums: fp32 atomics into grad_weight, or plain stores into this workgroup's
-    // partial image when a second kernel does the reduction.
-    block_sync();  // every wave is done with the rings; reuse the x ring as scratch
-    if (wave_active) {
-        float* scratch = reinterpret_cast<float*>(xring) + wg * 128;
+    // wave execute in order, so no barrier is needed inside the wave).  With TS > 1 the waves of
+    // one group then add their sums through LDS so that only one wave per group publishes:
+    // fp32 atomics into grad_weight, or plain stores into this workgroup's partial image when a
+    // second kernel does the reduction.
+    static_assert((WAVES * 128 + GB * (TS - 1) * NBLK * 128) * 4 <= (NRX * XROW_UNITS + NRD * DROW_UNITS) * 16,
+                  "reduction scratch does not fit in LDS");
+    block_sync();  // every wave is done with the rings; reuse them as scratch
+    {
+        float* scratch = reinterpret_cast<float*>(lds) + wave * 128;
+        float* red = reinterpret_cast<float*>(lds) + WAVES * 128;  // [group][ts-1][nb][e][32 lanes]
         const int k4 = 4 * ((lane >> 4) & 1);
         const int sj = (lane & 15) >> 3;
         const int c = lane & 7;
@@ -304,30 +324,59 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
 #endif
 #pragma unroll
         for (int r = 0; r < kR; ++r) {
+            float total[NBLK][4];
 #pragma unroll
             for (int nb = 0; nb < NBLK; ++nb) {
-                const int s = 2 * nb + sj;
                 if (lane >= 32) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) scratch[e * 32 + (lane - 32)] = acc[r + 1][nb][e];
                 }
-                if (lane < 32) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const float total = acc[r][nb][e] + scratch[e * 32 + lane];
-                        if (s < kS) {
+                for (int e = 0; e < 4; ++e) {
+                    total[nb][e] = 0.f;
+                    if (lane < 32) total[nb][e] = acc[r][nb][e] + scratch[e * 32 + lane];
+                }
+            }
+            if (TS > 1) {
+                if (ws > 0 && lane < 32) {
+#pragma unroll
+                    for (int nb = 0; nb < NBLK; ++nb)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            red[(((wg * (TS - 1) + ws - 1) * NBLK + nb) * 4 + e) * 32 + lane] = total[nb][e];
+                }
+                block_sync();
+                if (ws == 0 && lane < 32) {
+#pragma unroll
+                    for (int w2 = 0; w2 < TS - 1; ++w2)
+#pragma unroll
+                        for (int nb = 0; nb < NBLK; ++nb)
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                total[nb][e] += red[(((wg * (TS - 1) + w2) * NBLK + nb) * 4 + e) * 32 + lane];
+                }
+            }
+            if (wave_active && ws == 0 && lane < 32) {
+#pragma unroll
+                for (int nb = 0; nb < NBLK; ++nb) {
+                    const int s = 2 * nb + sj;
+                    if (s < kS) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
                             float* dst = out + (((long long)(8 * gglob + k4 + e) * kR + r) * kS + s) * 8 + c;
 #if SPIO_PARTIALS
-                            *dst = total;
+                            *dst = total[nb][e];
 #else
-                            atomic_add_f32(dst, total);
+                            atomic_add_f32(dst, total[nb][e]);
 #endif
                         }
                     }
                 }
             }
+            if (TS > 1) block_sync();  // the scratch is rewritten for the next filter row
         }
     }
+
 }
 
 #if SPIO_PARTIALS

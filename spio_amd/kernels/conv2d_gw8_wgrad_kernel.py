@@ -40,6 +40,8 @@ class Conv2dGw8WgradConfig:
         block_n_iters: image blocks a workgroup accumulates before its atomics.
         chunks: (direct variant only) pixel chunks per group.
         prefetch: rows of global loads in flight ahead of the computed row (even).
+        split: waves sharing the 32-pixel chunks of one group; their sums are added in LDS
+            before publishing, so bigger workgroups do not publish more.
         two_stage: 1 = workgroups store partial sums to a workspace and a second kernel
             reduces them; 0 = workgroups add into grad_weight with fp32 atomics.
         variant: "mfma" (row-streaming MFMA kernel) or "direct" (any shape).
@@ -53,12 +55,13 @@ class Conv2dGw8WgradConfig:
     variant: str = "mfma"
     prefetch: int = 2
     two_stage: int = 0
+    split: int = 1
 
 
 def wgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig) -> Dict[str, int]:
     """Host mirror of the compile-time constants of conv2d_gw8_wgrad_mfma.hip."""
     r, s = params.r, params.s
-    gb, bh, nb, iters = config.groups, config.block_h, config.block_n, config.block_n_iters
+    gb, bh, nb, iters, ts = config.groups, config.block_h, config.block_n, config.block_n_iters, config.split
     s2 = 2 * ((s + 1) // 2)
     wpi = params.q + s - 1
     f = nb * wpi
@@ -69,10 +72,12 @@ def wgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig) -> Dic
     fpd = 32 * kc
     gsd = fpd + ((9 - fpd % 16) + 16) % 16
     nrd = 2 * ((r + 2) // 2)
-    threads = 64 * gb
+    threads = 64 * gb * ts
+    lds_rings = (2 * gb * gsx + nrd * (gb * gsd + ((4 - (gb * gsd) % 16) + 16) % 16)) * 16
+    lds_scratch = (gb * ts * 128 + gb * (ts - 1) * (s2 // 2) * 128) * 4
     g = dict(
         NBLK=s2 // 2, ND=r + 1, WPI=wpi, F=f, KC=kc, GSX=gsx, GSD=gsd, NRD=nrd, THREADS=threads,
-        LDS_BYTES=(2 * gb * gsx + nrd * (gb * gsd + ((4 - (gb * gsd) % 16) + 16) % 16)) * 16,
+        LDS_BYTES=lds_rings, SCRATCH_BYTES=lds_scratch,
         LPTX=divup(f * gb, threads), LPTD=divup(nb * params.q * gb, threads),
         GBLKS=divup(params.groups, gb), PBLKS=divup(params.p, bh),
         NBLKS=divup(params.n, nb * iters), STEPS=bh + r - 1,
@@ -85,7 +90,9 @@ def wgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig) -> Dic
 def _mfma_config_is_legal(params, config) -> bool:
     g = wgrad_geometry(params, config)
     return (
-        config.groups <= MAX_WAVES
+        config.groups * config.split <= MAX_WAVES
+        and config.split <= g["KC"]
+        and g["SCRATCH_BYTES"] <= g["LDS_BYTES"]
         and config.block_h <= params.p
         and config.block_n * config.block_n_iters <= max(params.n, 1)
         and g["LDS_BYTES"] <= MAX_LDS_BYTES
@@ -137,10 +144,12 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None) -> List[Conv2dGw8Wgr
                         if pf > 2 and pf > bh + params.r - 1:
                             continue
                         for two_stage in (0, 1):
-                            cfg = Conv2dGw8WgradConfig(groups=gb, block_h=bh, block_n=nb, block_n_iters=iters,
-                                                       prefetch=pf, two_stage=two_stage)  # fmt: skip
-                            if _mfma_config_is_legal(params, cfg):
-                                found.append((_mfma_score(params, cfg, num_cus), cfg))
+                            for ts in (1, 2):
+                                cfg = Conv2dGw8WgradConfig(groups=gb, block_h=bh, block_n=nb,
+                                                           block_n_iters=iters, prefetch=pf,
+                                                           two_stage=two_stage, split=ts)  # fmt: skip
+                                if _mfma_config_is_legal(params, cfg):
+                                    found.append((_mfma_score(params, cfg, num_cus), cfg))
     found.sort(key=lambda sc: sc[0])
     configs = [cfg for _, cfg in found[:MAX_CONFIGS]]
     total_pix = params.n * params.p * params.q
@@ -164,7 +173,8 @@ def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig, _dev
     assert _mfma_config_is_legal(params, config), f"illegal configuration {config} for {params}"
     g = wgrad_geometry(params, config)
     defines.update(SPIO_GB=config.groups, SPIO_BH=config.block_h, SPIO_NB=config.block_n,
-                   SPIO_ITERS=config.block_n_iters, SPIO_PF=config.prefetch)  # fmt: skip
+                   SPIO_ITERS=config.block_n_iters, SPIO_PF=config.prefetch,
+                   SPIO_TS=config.split)  # fmt: skip
     spec = KernelSpec(defines, LaunchParams(grid=g["NUM_BLOCKS"], block=g["THREADS"]), MFMA_SOURCE, notes=g)
     if config.two_stage:
         num_partials = g["NBLKS"] * g["PBLKS"]

@@ -41,6 +41,7 @@ class KernelSpec:
     epilogue_launch_params: Optional[LaunchParams] = None
 
 
+
 class Kernel:
     """A compiled kernel bound to one device.  Made by KernelFactory.make_kernel."""
 
