@@ -96,6 +96,7 @@ constexpr int STEPS = BH + kR - 1;
 static_assert((NRX * XROW_UNITS + NRD * DROW_UNITS) * 16 <= 160 * 1024, "LDS overflow");
 static_assert(NRD % 2 == 0 && NRD >= kR + 1, "dy ring too small");
 static_assert(PF >= 2 && PF % 2 == 0, "prefetch distance must be even");
+constexpr int PART_WAVE_FLOATS = kR * NBLK * 4 * 32;  // floats one wave publishes (partial-block layout)
 
 
 SPIO_DEVICE spio_half8 read_tr_pair(const unsigned char* lo, const unsigned char* hi) {
@@ -308,17 +309,20 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
     // one group then add their sums through LDS so that only one wave per group publishes:
     // fp32 atomics into grad_weight, or plain stores into this workgroup's partial image when a
     // second kernel does the reduction.
-    static_assert((WAVES * 128 + GB * (TS - 1) * NBLK * 128) * 4 <= (NRX * XROW_UNITS + NRD * DROW_UNITS) * 16,
+    constexpr int SCRATCH_FLOATS = NBLK * 128;  // per wave
+    static_assert((WAVES * SCRATCH_FLOATS + GB * (TS - 1) * NBLK * 128) * 4 <= (NRX * XROW_UNITS + NRD * DROW_UNITS) * 16,
                   "reduction scratch does not fit in LDS");
     block_sync();  // every wave is done with the rings; reuse them as scratch
     {
-        float* scratch = reinterpret_cast<float*>(lds) + wave * 128;
-        float* red = reinterpret_cast<float*>(lds) + WAVES * 128;  // [group][ts-1][nb][e][32 lanes]
+        float* scratch = reinterpret_cast<float*>(lds) + wave * SCRATCH_FLOATS;
+        float* red = reinterpret_cast<float*>(lds) + WAVES * SCRATCH_FLOATS;  // [group][ts-1][nb][e][32 lanes]
         const int k4 = 4 * ((lane >> 4) & 1);
         const int sj = (lane & 15) >> 3;
         const int c = lane & 7;
 #if SPIO_PARTIALS
-        float* out = grad_weight + (long long)(nbk * PBLKS + pb) * ((long long)kC * kR * kS * 8);
+        // this wave's slice of the workgroup's partial block: [r][tap pair][e][32 lanes], so that
+        // every store instruction writes 128 contiguous bytes
+        float* out = grad_weight + (((long long)(nbk * PBLKS + pb) * GBLKS + cb) * GB + wg) * PART_WAVE_FLOATS;
 #else
         float* out = grad_weight;
 #endif
@@ -356,23 +360,35 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
                                 total[nb][e] += red[(((wg * (TS - 1) + w2) * NBLK + nb) * 4 + e) * 32 + lane];
                 }
             }
+#if SPIO_PARTIALS
+            // through the wave's LDS scratch once more so that all 64 lanes store 16 bytes each
+            if (wave_active && ws == 0) {
+                float* stage = scratch;  // NBLK * 128 floats: [tap pair][e][32 lanes]
+                if (lane < 32) {
+#pragma unroll
+                    for (int nb = 0; nb < NBLK; ++nb)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) stage[(nb * 4 + e) * 32 + lane] = total[nb][e];
+                }
+                const spio_float4* stage4 = reinterpret_cast<const spio_float4*>(stage);
+                spio_float4* out4 = reinterpret_cast<spio_float4*>(out) + r * NBLK * 32;
+#pragma unroll
+                for (int i = lane; i < NBLK * 32; i += 64) __builtin_nontemporal_store(stage4[i], out4 + i);
+            }
+#else
             if (wave_active && ws == 0 && lane < 32) {
 #pragma unroll
                 for (int nb = 0; nb < NBLK; ++nb) {
                     const int s = 2 * nb + sj;
                     if (s < kS) {
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            float* dst = out + (((long long)(8 * gglob + k4 + e) * kR + r) * kS + s) * 8 + c;
-#if SPIO_PARTIALS
-                            *dst = total[nb][e];
-#else
-                            atomic_add_f32(dst, total[nb][e]);
-#endif
-                        }
+                        for (int e = 0; e < 4; ++e)
+                            atomic_add_f32(out + (((long long)(8 * gglob + k4 + e) * kR + r) * kS + s) * 8 + c,
+                                           total[nb][e]);
                     }
                 }
             }
+#endif
             if (TS > 1) block_sync();  // the scratch is rewritten for the next filter row
         }
     }
@@ -380,28 +396,57 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
 }
 
 #if SPIO_PARTIALS
-// Second stage: grad_weight[e] += sum over partial images.  Thread (column of 4 floats,
-// slice) adds the partial images p = slice, slice + SLICES, ... and publishes with atomics, so
-// the result accumulates onto whatever grad_weight holds, like the single-stage kernel.
-#ifndef SPIO_REDUCE_SLICES
-#define SPIO_REDUCE_SLICES 1
-#endif
+// Second stage: grad_weight += sum over the partial blocks.  A workgroup owns 8 float4 columns
+// of one channel block (128 contiguous bytes of every partial block); its 32 slices each add the
+// blocks p = slice, slice + 32, ... with 8 loads in flight, the slices are added through LDS and
+// slice 0 adds the total onto grad_weight.  Every element of grad_weight has exactly one owner,
+// so no atomics are needed and the sum does not depend on timing.  A column is four consecutive
+// lanes of the publishing wave, i.e. four consecutive channels c of one (k, r, s).
 #define SPIO_CONCAT2(a, b) a##b
 #define SPIO_CONCAT(a, b) SPIO_CONCAT2(a, b)
 extern "C" __global__ void SPIO_LAUNCH_BOUNDS(256)
 SPIO_CONCAT(SPIO_KERNEL_NAME, _reduce)(float* __restrict__ grad_weight, const spio_float4* __restrict__ partials) {
-    constexpr int COLS = kC * kR * kS * 2;  // float4 columns of one image
+    constexpr int BLOCK_F4 = GB * PART_WAVE_FLOATS / 4;  // float4 columns of one partial block
     constexpr int NPART = NBLKS * PBLKS;
-    constexpr int SLICES = SPIO_REDUCE_SLICES;
-    const int idx = block_id() * 256 + thread_id();
-    if (idx >= COLS * SLICES) return;
-    const int col = idx % COLS;
-    const int slice = idx / COLS;
+    constexpr int SLICES = 32;
+    constexpr int UN = 8;
+    __shared__ spio_float4 red[SLICES][8];
+    const int tid = thread_id();
+    const int cl = tid & 7;
+    const int slice = tid >> 3;
+    const int col = (block_id() % (BLOCK_F4 / 8)) * 8 + cl;
+    const int cb = block_id() / (BLOCK_F4 / 8);
     spio_float4 sum = spio_float4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-    for (int p = slice; p < NPART; p += SLICES) sum += partials[(long long)p * COLS + col];
-    float* dst = grad_weight + 4 * (long long)col;
+    for (int base = slice; base < NPART; base += SLICES * UN) {
+        spio_float4 v[UN];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) atomic_add_f32(dst + e, sum[e]);
+        for (int i = 0; i < UN; ++i) {
+            const int p = base + i * SLICES;
+            v[i] = spio_float4{0.f, 0.f, 0.f, 0.f};
+            if (p < NPART) v[i] = partials[((long long)p * GBLKS + cb) * BLOCK_F4 + col];
+        }
+#pragma unroll
+        for (int i = 0; i < UN; ++i) sum += v[i];
+    }
+    red[slice][cl] = sum;
+    block_sync();
+    if (slice == 0) {
+#pragma unroll 4
+        for (int i = 1; i < SLICES; ++i) sum += red[i][cl];
+        // float index inside the block -> (group, r, tap pair, e, lane)
+        const int f = 4 * col;
+        const int l32 = f & 31;
+        const int e = (f >> 5) & 3;
+        const int rn = (f >> 7) % (kR * NBLK);
+        const int g = (f >> 7) / (kR * NBLK);
+        const int r = rn / NBLK;
+        const int s = 2 * (rn % NBLK) + ((l32 & 15) >> 3);
+        const int k = 8 * (cb * GB + g) + 4 * (l32 >> 4) + e;
+        if (cb * GB + g < kGroups && s < kS) {
+            spio_float4* dst =
+                reinterpret_cast<spio_float4*>(grad_weight + (((long long)k * kR + r) * kS + s) * 8 + (l32 & 7));
+            *dst = *dst + sum;
+        }
+    }
 }
 #endif

@@ -26,7 +26,6 @@ MAX_LDS_BYTES = 96 * 1024
 MAX_LOADS_PER_THREAD = 8
 MAX_ACCUMULATORS = 32
 MAX_CONFIGS = 32
-REDUCE_TARGET_THREADS = 64 * 1024
 
 
 @dataclass(frozen=True)
@@ -74,7 +73,7 @@ def wgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig) -> Dic
     nrd = 2 * ((r + 2) // 2)
     threads = 64 * gb * ts
     lds_rings = (2 * gb * gsx + nrd * (gb * gsd + ((4 - (gb * gsd) % 16) + 16) % 16)) * 16
-    lds_scratch = (gb * ts * 128 + gb * (ts - 1) * (s2 // 2) * 128) * 4
+    lds_scratch = (gb * ts * (s2 // 2) * 128 + gb * (ts - 1) * (s2 // 2) * 128) * 4
     g = dict(
         NBLK=s2 // 2, ND=r + 1, WPI=wpi, F=f, KC=kc, GSX=gsx, GSD=gsd, NRD=nrd, THREADS=threads,
         LDS_BYTES=lds_rings, SCRATCH_BYTES=lds_scratch,
@@ -178,12 +177,14 @@ def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig, _dev
     spec = KernelSpec(defines, LaunchParams(grid=g["NUM_BLOCKS"], block=g["THREADS"]), MFMA_SOURCE, notes=g)
     if config.two_stage:
         num_partials = g["NBLKS"] * g["PBLKS"]
-        cols = params.c * params.r * params.s * 2  # float4 columns of one partial image
-        slices = max(1, min(num_partials, divup(REDUCE_TARGET_THREADS, cols)))
-        defines.update(SPIO_PARTIALS=1, SPIO_REDUCE_SLICES=slices)
+        # float4 columns of the partial blocks of one (image block, row block): per wave
+        # [r][tap pair][4][32 lanes] floats
+        cols = g["GBLKS"] * config.groups * params.r * g["NBLK"] * 32
+        defines.update(SPIO_PARTIALS=1)
         spec.workspace_bytes = num_partials * cols * 16
         spec.epilogue_suffix = "_reduce"
-        spec.epilogue_launch_params = LaunchParams(grid=divup(cols * slices, 256), block=256)
+        # one workgroup per 8 float4 columns (cols is a multiple of 8 per channel block)
+        spec.epilogue_launch_params = LaunchParams(grid=cols // 8, block=256)
     return spec
 
 
