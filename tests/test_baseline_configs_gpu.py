@@ -1,0 +1,123 @@
+"""The benchmark configurations at their full sizes, through the operator (tuned kernels are
+used when a record exists, else the first configuration), against the fp32 CPU oracle, plus
+size-independent properties (bilinearity / adjoint identities evaluated from the GPU results) and
+the ConvNeXt-shaped network.  GPU only."""
+
+import pytest
+import torch
+
+from convnext_gw8 import ConvNeXtGw8
+from helpers import to_gpu
+from oracle import conv2d_gw8_oracle as oracle
+from spio_amd.functional import conv2d_gw8
+from spio_amd.kernels import Conv2dGw8Params, Conv2dStats
+from spio_amd.layers import Conv2dGw8
+from spio_amd.transform import transform
+
+pytestmark = pytest.mark.gpu
+
+CONFIGS = {
+    "cfg1": (Conv2dGw8Params(n=32, c=64, h=56, w=56, padding=1), 0),
+    "cfg2": (Conv2dGw8Params(n=128, c=128, h=28, w=28, padding=1), 1),
+    "cfg3": (Conv2dGw8Params(n=256, c=256, h=14, w=14, padding=3, r=7, s=7), 2),
+    "target": (Conv2dGw8Params(n=128, c=64, h=56, w=56, padding=1), 0),
+}
+
+
+def _run(params, seed):
+    x, w, _b, dy = oracle.make_args(params.n, params.c, params.h, params.w, params.r, params.s,
+                                    params.padding_h, params.padding_w, False, seed, weight_init="kaiming")  # fmt: skip
+    xg, wg, dyg = to_gpu(x).requires_grad_(True), to_gpu(w).requires_grad_(True), to_gpu(dy)
+    y = conv2d_gw8(xg, wg, None, stride=1, padding_y=params.padding_h, padding_x=params.padding_w,
+                   groups=params.groups)  # fmt: skip
+    dx, dw, _none = torch.ops.spio.conv2d_gw8_backward(xg.detach(), wg.detach(), None, dyg, params.padding_h,
+                                                       params.padding_w, True, True, False)  # fmt: skip
+    torch.cuda.synchronize()
+    return x, w, dy, y.detach(), dx, dw
+
+
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_full_size_against_oracle(name):
+    """North-star tolerance (rel 2e-3 / atol 1e-2 on fp16 outputs) and the reference's
+    accumulation-depth tolerance, at the benchmark size."""
+    params, seed = CONFIGS[name]
+    x, w, dy, y, dx, dw = _run(params, seed)
+    depth = Conv2dStats(params, output_names=["output", "grad_input", "grad_weight"]).accumulation_depths
+    y_e = oracle.fprop_torch(x, w, None, params.padding_h, params.padding_w)
+    oracle.check_close(y, y_e, what=f"{name} fprop (north-star tolerance)")
+    oracle.check_close(y, y_e, acc_depth=depth[0], what=f"{name} fprop")
+    dx_e, dw_e, _ = oracle.grads_torch(x, w, None, dy, params.padding_h, params.padding_w)
+    oracle.check_close(dx, dx_e, what=f"{name} dgrad (north-star tolerance)")
+    oracle.check_close(dx, dx_e, acc_depth=depth[1], what=f"{name} dgrad")
+    assert dw.dtype == torch.float32
+    oracle.check_close(dw, dw_e, acc_depth=depth[2], what=f"{name} wgrad")
+
+
+@pytest.mark.parametrize("name", ["cfg2", "cfg3"])
+def test_adjoint_identities_from_gpu_results(name):
+    """<conv(x), dy> == <x, dgrad(dy)> == <w, wgrad(x, dy)>, evaluated in fp64 from what the
+    kernels returned.  y and dx are rounded to fp16, so the identities hold to ~1e-3 relative."""
+    params, seed = CONFIGS[name]
+    x, w, dy, y, dx, dw = _run(params, seed)
+    lhs = float((y.double().cpu() * dy.double()).sum())
+    via_dx = float((dx.double().cpu() * x.double()).sum())
+    via_dw = float((dw.double().cpu() * w.double()).sum())
+    scale = float((y.double().cpu().abs() * dy.double().abs()).sum())
+    assert abs(lhs - via_dx) <= 2e-3 * scale * 1e-1
+    assert abs(lhs - via_dw) <= 2e-3 * scale * 1e-1
+    assert abs(via_dx - via_dw) <= 2e-3 * scale * 1e-1
+
+
+def test_forward_is_linear_in_the_input_at_full_size():
+    """conv(a + b) == conv(a) + conv(b) up to the output rounding, at the benchmark size."""
+    params, seed = CONFIGS["target"]
+    a, w, _b, _dy = oracle.make_args(params.n, params.c, params.h, params.w, 3, 3, 1, 1, False, seed)
+    b = oracle.make_args(params.n, params.c, params.h, params.w, 3, 3, 1, 1, False, seed + 1)[0]
+    ag, bg, wg = to_gpu(a), to_gpu(b), to_gpu(w)
+    sg = (ag.float() + bg.float()).half()  # the sum itself is rounded: compare against conv of that
+    call = lambda t: conv2d_gw8(t, wg, None, 1, 1, 1, 1, params.groups).float()
+    lhs = call(sg)
+    rhs = call(ag) + call(bg)
+    # |x| <= 6, 72 products with |w| <= 0.12: the rounding of s and of the three outputs stays
+    # far below this bound
+    assert float((lhs - rhs).abs().max()) < 0.05
+    assert float((lhs - rhs).abs().mean()) < 2e-3
+
+
+def test_batch_sweep_shapes_small_batches():
+    """Forward at C=64, 56x56 for the small-batch end of the sweep (N = 1 .. 16)."""
+    for n in (1, 2, 4, 8, 16):
+        params = Conv2dGw8Params(n=n, c=64, h=56, w=56, padding=1)
+        x, w, _b, _dy = oracle.make_args(n, 64, 56, 56, 3, 3, 1, 1, False, 0, weight_init="kaiming")
+        y = conv2d_gw8(to_gpu(x), to_gpu(w), None, 1, 1, 1, 1, 8)
+        oracle.check_close(y, oracle.fprop_torch(x, w, None, 1, 1), acc_depth=72, what=params.encode())
+
+
+def test_convnext_shaped_network_logits():
+    """The network of the fifth configuration: logits of the fp16 GPU model with Conv2dGw8
+    layers against the same weights in fp32 on the CPU with nn.Conv2d(groups=C/8).  Batch 4
+    keeps the CPU side to seconds; every gw8 convolution shape of the full-batch run occurs."""
+    torch.manual_seed(3)
+    cpu_model = ConvNeXtGw8().eval()
+    images = torch.randn(4, 3, 224, 224).half().float()
+    with torch.no_grad():
+        want = cpu_model(images)
+    gpu_model = transform(ConvNeXtGw8().eval())
+    gpu_model.load_state_dict(cpu_model.state_dict())
+    assert sum(isinstance(m, Conv2dGw8) for m in gpu_model.modules()) == 18
+    gpu_model = gpu_model.cuda().to(memory_format=torch.channels_last)
+    with torch.no_grad(), torch.autocast(device_type="cuda", dtype=torch.float16):
+        got = gpu_model(images.cuda().contiguous(memory_format=torch.channels_last))
+    got = got.float().cpu()
+    # 18 residual blocks in fp16 against fp32: logits are O(1); agree to a few 1e-2 and rank alike
+    assert float((got - want).abs().max()) < 0.08 * max(1.0, float(want.abs().max()))
+    assert torch.equal(got.argmax(dim=1), want.argmax(dim=1))
+    # ... and a wrong convolution would show: zeroing one conv's weights moves the logits
+    first = next(m for m in gpu_model.modules() if isinstance(m, Conv2dGw8))
+    with torch.no_grad():
+        saved = first.weight.clone()
+        first.weight.zero_()
+        with torch.autocast(device_type="cuda", dtype=torch.float16):
+            moved = gpu_model(images.cuda().contiguous(memory_format=torch.channels_last)).float().cpu()
+        first.weight.copy_(saved)
+    assert float((moved - want).abs().max()) > 10 * float((got - want).abs().max())
