@@ -32,6 +32,14 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what
+# the same counter reads for the plain copy kernel (profiles/conv2d_gw8_target_hbm_traffic.md).
+MEASURED_TRAFFIC_BYTES = {
+    ("target", "fprop"): 103_670_000,
+    ("target", "dgrad"): 103_650_000,
+    ("target", "wgrad"): 105_890_000,
+}
 CACHE_BYTES = 256 * 1024 * 1024
 
 WORKLOADS = {
@@ -244,7 +252,7 @@ def main():
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": kernels[dominant]["frac_of_hbm_peak"],
-        "traffic": None,
+        "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, dominant)),
     }
 
     result = {
