@@ -148,12 +148,20 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
     const bool wave_active = gglob < kGroups;
 
     // ---- loop-invariant addressing of the cooperative row load ----
-    int in_off[LPT];   // 16-byte units from src; row term excluded; -1 = zero cell
+    // Every thread issues the same number of loads on every step, without branches, so that the
+    // compiler can count outstanding loads exactly and wait only for the row it needs (a load
+    // under a branch makes it wait for all of them).  Cells that hold no source data (halo
+    // columns, missing images or groups) load a valid dummy address and are zeroed when the row
+    // is written to LDS.
+    int in_off[LPT];   // 16-byte units from src; row term excluded
+    bool in_ok[LPT];   // the cell carries source data
     int in_lds[LPT];   // 16-byte unit inside a ring row; -1 = no cell
+    const int dummy_off = n0 * SH * SW * kGroups;  // first unit of the workgroup's first image
 #pragma unroll
     for (int l = 0; l < LPT; ++l) {
         const int cell = tid + THREADS * l;
-        in_off[l] = -1;
+        in_off[l] = dummy_off;
+        in_ok[l] = false;
         in_lds[l] = -1;
         if (cell < IN_CELLS) {
             const int g = cell % GB;
@@ -161,8 +169,10 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
             const int img = f / WPI;
             const int col = f % WPI - EPX;
             in_lds[l] = g * GS + f;
-            if (col >= 0 && col < SW && n0 + img < kN && cb * GB + g < kGroups)
+            if (col >= 0 && col < SW && n0 + img < kN && cb * GB + g < kGroups) {
                 in_off[l] = ((n0 + img) * SH * SW + col) * kGroups + cb * GB + g;
+                in_ok[l] = true;
+            }
         }
     }
     // ---- loop-invariant addressing of the cooperative row store ----
@@ -282,13 +292,10 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
     spio_uint4 pre[PF][LPT];
 #pragma unroll
     for (int t = 0; t < PF; ++t) {
-        const int h = p0 + t - EPY;
-        const bool row_ok = t < STEPS && h >= 0 && h < SH;
+        // rows outside the image are loaded from the nearest real row and never used
+        const int h = imin(imax(p0 + t - EPY, 0), SH - 1);
 #pragma unroll
-        for (int l = 0; l < LPT; ++l) {
-            pre[t][l] = spio_uint4{0u, 0u, 0u, 0u};
-            if (row_ok && in_off[l] >= 0) pre[t][l] = load_row(src + in_off[l] + h * row_units, t);
-        }
+        for (int l = 0; l < LPT; ++l) pre[t][l] = load_row(src + in_off[l] + h * row_units, t);
     }
     block_sync();  // ring zeroed
     {
@@ -296,10 +303,26 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
         if (h >= 0 && h < SH) {
 #pragma unroll
             for (int l = 0; l < LPT; ++l)
-                if (in_lds[l] >= 0) ring[in_lds[l]] = pre[0][l];
+                if (in_lds[l] >= 0) ring[in_lds[l]] = in_ok[l] ? pre[0][l] : spio_uint4{0u, 0u, 0u, 0u};
         }
     }
     block_sync();
+
+    // Coalesced store of the output row staged at step `ts` (in stage buffer `obuf`): the row
+    // that received its last tap at that step.  Called one step later, after the barrier.
+    auto store_output_row = [&](int ts, int obuf) {
+        const int p = p0 + ts - (kR - 1);
+        if (ts >= kR - 1 && p < DH) {
+#pragma unroll
+            for (int s = 0; s < SPT; ++s) {
+                if (out_off[s] >= 0) {
+                    const spio_uint4 v =
+                        *reinterpret_cast<const spio_uint4*>(ostage + obuf * OUT_ROW_BYTES + out_lds[s]);
+                    store_stream(v, dst + out_off[s] + p * dst_row_units);
+                }
+            }
+        }
+    };
 
     for (int tb = 0; tb < STEPS; tb += UNROLL) {
 #pragma unroll
@@ -316,38 +339,47 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
             // 1. prefetch source row t+PF (its register buffer is free: row t is in LDS)
             {
                 const int tt = t + PF;
-                const int h = p0 + tt - EPY;
-                const bool row_ok = tt < STEPS && h >= 0 && h < SH;
+                if (PF < STEPS) {  // compile-time: with PF >= STEPS the prologue loaded every row
+                    // past the last row the loads repeat it (cache hits) and are never used
+                    const int h = imin(imax(p0 + imin(tt, STEPS - 1) - EPY, 0), SH - 1);
 #pragma unroll
-                for (int l = 0; l < LPT; ++l) {
-                    spio_uint4 v = spio_uint4{0u, 0u, 0u, 0u};
-                    if (row_ok && in_off[l] >= 0) v = load_row(src + in_off[l] + h * row_units, tt);
-                    pre[pbuf][l] = v;
+                    for (int l = 0; l < LPT; ++l) pre[pbuf][l] = load_row(src + in_off[l] + h * row_units, tt);
                 }
             }
 
-            // 2. multiply source row t into the live output rows
+            // 2. multiply source row t into the live output rows.  The fragment reads are issued
+            //    first; the previous step's output row is stored while they are in flight.
             const int hcur = p0 + t - EPY;
-            if (wave_active && hcur >= 0 && hcur < SH) {
+            const bool row_live = wave_active && hcur >= 0 && hcur < SH;
+            spio_half8 bfrag[TPW][KB];
+            if (row_live) {
                 const spio_uint4* rrow = ring + rbuf * RING_ROW_UNITS + wg * GS + (lane & 15) + (lane >> 4);
 #pragma unroll
                 for (int i = 0; i < TPW; ++i) {
                     const int tile = ws + TS * i;
                     if (TS == 1 || tile < WT) {
-                        spio_half8 bfrag[KB];
 #pragma unroll
                         for (int u = 0; u < KB; ++u) {
                             Pack16 v;
                             v.u = rrow[16 * tile + 4 * u];
-                            bfrag[u] = v.h;
+                            bfrag[i][u] = v.h;
                         }
+                    }
+                }
+            }
+            store_output_row(t - 1, (uu + 1) & 1);
+            if (row_live) {
+#pragma unroll
+                for (int i = 0; i < TPW; ++i) {
+                    const int tile = ws + TS * i;
+                    if (TS == 1 || tile < WT) {
 #pragma unroll
                         for (int a = 0; a < NACC; ++a) {
                             const int d = pmod(ph - 2 * a, NS);
 #pragma unroll
                             for (int u = 0; u < KB; ++u)
                                 acc[i][a] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                                    wfrag[d][u], bfrag[u], acc[i][a], 0, 0, 0);
+                                    wfrag[d][u], bfrag[i][u], acc[i][a], 0, 0, 0);
                         }
                     }
                 }
@@ -385,26 +417,15 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
                 if (t + 1 < STEPS && hn >= 0 && hn < SH) {
 #pragma unroll
                     for (int l = 0; l < LPT; ++l)
-                        if (in_lds[l] >= 0) ring[((uu + 1) % NR) * RING_ROW_UNITS + in_lds[l]] = pre[(uu + 1) % PF][l];
+                        if (in_lds[l] >= 0)
+                            ring[((uu + 1) % NR) * RING_ROW_UNITS + in_lds[l]] =
+                                in_ok[l] ? pre[(uu + 1) % PF][l] : spio_uint4{0u, 0u, 0u, 0u};
                 }
             }
 
             block_sync();
 
-            // 5. coalesced store of the staged output row
-            {
-                const int p = p0 + t - (kR - 1);
-                if (t >= kR - 1 && p < DH) {
-#pragma unroll
-                    for (int s = 0; s < SPT; ++s) {
-                        if (out_off[s] >= 0) {
-                            const spio_uint4 v = *reinterpret_cast<const spio_uint4*>(
-                                ostage + obuf * OUT_ROW_BYTES + out_lds[s]);
-                            store_stream(v, dst + out_off[s] + p * dst_row_units);
-                        }
-                    }
-                }
-            }
         }
     }
+    store_output_row(STEPS - 1, (STEPS - 1) & 1);  // the last row
 }
