@@ -15,6 +15,9 @@ The single JSON line printed at the end reports
   kernels    per-kernel us, effective GB/s and fraction of the 8 TB/s roofline,
              timed with HIP events on the launch stream,
   roofline   the same for the kernel that takes the most time,
+  copy_yardstick  a plain non-temporal copy of the same volume (what HBM gives a read-X/write-X
+             kernel on this device),
+  torch_gpu_conv2d  torch's own grouped conv2d (MIOpen) on the same GPU and shapes,
   cpu_baseline  the reference's CPU oracle path (torch conv2d fp32, groups=C/8,
              and its autograd) on the host cores for a bounded sample.
 
@@ -62,6 +65,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="target", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-torch-gpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-batch", type=int, default=8)
     return ap.parse_args()
 
@@ -114,6 +118,48 @@ def copy_yardstick(nbytes, nsets, device, iters):
         "note": "plain non-temporal copy of one activation tensor in and one out: the HBM rate "
                 "a read-X/write-X kernel reaches on this device",
     }
+
+
+def torch_gpu_conv2d(params, sets, w, iters):
+    """The framework's own grouped conv2d on the same GPU (MIOpen through torch), fp16
+    channels_last, same shapes: the comparison the reference draws against PyTorch/cuDNN
+    (figures/batch_size_vs_eff_bandwidth__*.png).  torch.cuda events on the current stream."""
+    import torch
+    import torch.nn.functional as F
+
+    pad = (params.padding_h, params.padding_w)
+    out = {}
+    try:
+        x0 = sets[0]["x"].detach().requires_grad_(True)
+        w0 = w.detach().requires_grad_(True)
+        y0 = F.conv2d(x0, w0, None, 1, pad, 1, params.groups)
+
+        def fwd(i):
+            F.conv2d(sets[i % len(sets)]["x"], w, None, 1, pad, 1, params.groups)
+
+        def dgrad(i):
+            torch.autograd.grad(y0, x0, sets[i % len(sets)]["dy"], retain_graph=True)
+
+        def wgrad(i):
+            torch.autograd.grad(y0, w0, sets[i % len(sets)]["dy"], retain_graph=True)
+
+        for name, fn in (("fprop", fwd), ("dgrad", dgrad), ("wgrad", wgrad)):
+            for i in range(3):
+                fn(i)
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            start.record()
+            for i in range(iters):
+                fn(i)
+            stop.record()
+            torch.cuda.synchronize()
+            out[name + "_us"] = round(start.elapsed_time(stop) * 1e3 / iters, 2)
+        out["note"] = ("torch.nn.functional.conv2d(groups=C/8) fp16 channels_last and its autograd on the "
+                       "same GPU; dgrad/wgrad call torch.autograd.grad on one saved graph (input rotates only "
+                       "for the upstream gradient)")
+    except Exception as e:  # pylint: disable=broad-except
+        out["error"] = f"{type(e).__name__}: {e}"[:200]
+    return out
 
 
 def cpu_baseline(params_kwargs, seed, sample_batch):
@@ -278,6 +324,8 @@ def main():
         "kernels": kernels,
         "roofline": roofline,
     }
+    if not args.no_torch_gpu_baseline:
+        result["torch_gpu_conv2d"] = torch_gpu_conv2d(params, sets, w, min(iters, 50))
     del arg_sets
     del sets
     torch.cuda.empty_cache()

@@ -22,7 +22,7 @@ DIRECT_SOURCE = "conv2d_gw8_direct.hip"
 MFMA_SOURCE = "conv2d_gw8_wgrad_mfma.hip"
 
 MAX_WAVES = 16
-MAX_LDS_BYTES = 96 * 1024
+MAX_LDS_BYTES = 128 * 1024
 MAX_LOADS_PER_THREAD = 8
 MAX_ACCUMULATORS = 32
 MAX_CONFIGS = 32

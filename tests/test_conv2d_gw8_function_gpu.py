@@ -163,3 +163,38 @@ def test_opcheck():
     args = (to_gpu(x).requires_grad_(True), to_gpu(w).requires_grad_(True), to_gpu(b).requires_grad_(True))
     kwargs = dict(stride=1, padding_y=1, padding_x=1, dilation=1, groups=p.groups)
     torch.library.opcheck(conv2d_gw8, args, kwargs)
+
+
+def test_compiled_training_step():
+    """torch.compile of a layer, forward and backward: the fake implementations of both ops
+    (shapes, strides, fp32 grad_weight) must agree with what the real ops return."""
+    torch.manual_seed(2)
+    layer = Conv2dGw8(32, 32, 3, padding=1, groups=4).cuda().to(memory_format=torch.channels_last)
+    compiled = torch.compile(layer)
+    x = torch.randn(2, 32, 10, 12, device="cuda").contiguous(memory_format=torch.channels_last).requires_grad_(True)
+    with torch.autocast(device_type="cuda", dtype=torch.float16):
+        y = compiled(x)
+    dy = torch.randn_like(y)
+    y.backward(dy)
+    dx_e, dw_e, db_e = oracle.grads_torch(x.detach().half(), layer.weight.detach().half(), layer.bias.detach(),
+                                          dy.half(), 1, 1)  # fmt: skip
+    oracle.check_close(x.grad, dx_e, acc_depth=72, what="compiled dx")
+    oracle.check_close(layer.weight.grad, dw_e, acc_depth=2 * 10 * 12, what="compiled dw")
+    oracle.check_close(layer.bias.grad, db_e, acc_depth=2 * 10 * 12, what="compiled db")
+
+
+def test_kernel_launch_argument_errors():
+    """Launch-time checks raise ValueError, as the reference's Kernel.launch does
+    (spio/kernels/kernel.py:135-151): tensors that are not channels_last, CPU tensors."""
+    from spio_amd.kernels import conv2d_gw8_kernel_factory
+
+    p = Conv2dGw8Params(n=2, c=16, h=8, w=8)
+    x, w, _b, _dy = oracle.make_args(p.n, p.c, p.h, p.w, 3, 3, 1, 1, False, 0)
+    kernel = conv2d_gw8_kernel_factory.get_kernel(p, torch.device("cuda", 0))
+    out = torch.empty(p.output_shape, device="cuda", dtype=torch.float16).contiguous(memory_format=torch.channels_last)
+    with pytest.raises(ValueError, match="Error in kernel"):
+        kernel(out, x.contiguous().cuda(), to_gpu(w), None)  # NCHW-contiguous input
+    with pytest.raises(ValueError, match="Error in kernel"):
+        kernel(out, x, to_gpu(w), None)  # CPU tensor among GPU tensors
+    kernel(out, to_gpu(x), to_gpu(w), None)  # and the right call still works
+    oracle.check_close(out, oracle.fprop_torch(x, w, None, 1, 1), acc_depth=72, what="after errors")
