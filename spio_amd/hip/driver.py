@@ -9,6 +9,7 @@ like the reference's driver errors (driver.pyx:118-123).
 
 import ctypes
 import os
+import struct
 import threading
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
@@ -69,6 +70,8 @@ class DeviceAttributes:
 # Exported symbols and their ctypes signatures; also used by the tests that
 # check the library against the header.
 _vp = ctypes.c_void_p
+_F32_BITS = struct.Struct("<f")  # a float argument travels as its IEEE-754 single bits
+_F32 = struct.Struct("<I")
 _SIGNATURES = {
     "spio_hip_init": ([ctypes.c_char_p, ctypes.c_char_p], ctypes.c_int),
     "spio_hip_last_error": ([], ctypes.c_char_p),
@@ -271,44 +274,49 @@ class Function:
         _check(_lib.spio_hip_func_set_max_dynamic_lds(self._handle, int(nbytes)))
 
     @staticmethod
-    def marshal(args) -> Tuple[object, list]:
+    def marshal(args) -> Tuple[object, object]:
         """Convert launch arguments to the `params` array of the C ABI.
 
         Follows the reference's conventions (driver.pyx:181-199): tensors pass
         their device pointer, None a null pointer, int a 64-bit integer, float
-        a 32-bit float.  Returns the ctypes array and the objects that must be
+        a 32-bit float.  Every value sits in its own 8-byte slot of one array
+        (a 32-bit float in the low bytes of its slot) and `params[i]` is the
+        address of slot i.  Returns `params` and the slot array, which must be
         kept alive until the launch call returns.
         """
-        if len(args) > Function.MAX_ARGS:
-            raise ValueError(f"Too many kernel arguments: {len(args)} > {Function.MAX_ARGS}")
-        storage = []
+        n = len(args)
+        if n > Function.MAX_ARGS:
+            raise ValueError(f"Too many kernel arguments: {n} > {Function.MAX_ARGS}")
+        slots = []
         for a in args:
             if a is None:
-                storage.append(ctypes.c_void_p(0))
+                slots.append(0)
             elif hasattr(a, "data_ptr"):
-                storage.append(ctypes.c_void_p(a.data_ptr()))
+                slots.append(a.data_ptr())
             elif isinstance(a, bool):
                 raise ValueError(f"Unsupported kernel argument type: {type(a)}")
             elif isinstance(a, int):
-                storage.append(ctypes.c_longlong(a))
+                if not -(1 << 63) <= a < (1 << 64):
+                    raise ValueError(f"Integer kernel argument out of 64-bit range: {a}")
+                slots.append(a & 0xFFFFFFFFFFFFFFFF)
             elif isinstance(a, float):
-                storage.append(ctypes.c_float(a))
+                slots.append(_F32.unpack(_F32_BITS.pack(a))[0])
             else:
                 raise ValueError(f"Unsupported kernel argument type: {type(a)}")
-        arr = (_vp * max(len(storage), 1))(
-            *[ctypes.cast(ctypes.pointer(s), _vp) for s in storage]
-        )
-        return arr, storage
+        values = (ctypes.c_uint64 * max(n, 1))(*slots)
+        base = ctypes.addressof(values)
+        params = (_vp * max(n, 1))(*range(base, base + 8 * max(n, 1), 8))
+        return params, values
 
     def launch(self, grid, block, args, shared_mem_bytes: int = 0, stream: int = 0):
         """Asynchronous launch on `stream` (an integer hipStream_t, 0 = null)."""
-        arr, keep = self.marshal(args)
-        _check(
-            _lib.spio_hip_launch(
-                self._handle, grid[0], grid[1], grid[2], block[0], block[1], block[2],
-                int(shared_mem_bytes), stream or None, arr, len(keep),
-            )  # fmt: skip
-        )
+        params, _values = self.marshal(args)
+        rc = _lib.spio_hip_launch(
+            self._handle, grid[0], grid[1], grid[2], block[0], block[1], block[2],
+            shared_mem_bytes, stream or None, params, len(args),
+        )  # fmt: skip
+        if rc:
+            _check(rc)
 
     def launch_timed(
         self, grid, block, arg_sets: List[Sequence], shared_mem_bytes: int = 0, stream: int = 0,

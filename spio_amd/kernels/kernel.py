@@ -99,6 +99,7 @@ class Kernel:
         self.epilogue_function = None
 
     def _prepare(self, args):
+        """Check the arguments and return the device they live on."""
         if self.function is None:
             raise ValueError("kernel is not loaded")
         if self.args_checker is not None:
@@ -108,25 +109,26 @@ class Kernel:
             if isinstance(a, torch.Tensor) and a.numel() > 0:
                 if device is None:
                     device = a.device
-                assert a.device == device, "Not all tensor arguments are on the same device"
+                elif a.device != device:
+                    raise AssertionError("Not all tensor arguments are on the same device")
         if device is None or device.type != "cuda":
             raise ValueError("kernel arguments must be GPU tensors")
-        return device, [a.detach() if isinstance(a, torch.Tensor) else a for a in args]
+        return device
 
     def launch(self, *args):
         """Asynchronous launch on torch's current stream of the arguments' device."""
         try:
-            device, kargs = self._prepare(args)
+            device = self._prepare(args)
             spec = self.kernel_spec
             lp = spec.launch_params
             stream = torch.cuda.current_stream(device).cuda_stream
             if self.epilogue_function is None:
-                self.function.launch(lp.grid, lp.block, kargs, lp.shared_mem_bytes, stream)
+                self.function.launch(lp.grid, lp.block, args, lp.shared_mem_bytes, stream)
             else:
                 workspace = self._workspace(device)
-                self.function.launch(lp.grid, lp.block, [workspace] + kargs[1:], lp.shared_mem_bytes, stream)
+                self.function.launch(lp.grid, lp.block, (workspace,) + args[1:], lp.shared_mem_bytes, stream)
                 ep = spec.epilogue_launch_params
-                self.epilogue_function.launch(ep.grid, ep.block, [kargs[0], workspace], ep.shared_mem_bytes, stream)
+                self.epilogue_function.launch(ep.grid, ep.block, (args[0], workspace), ep.shared_mem_bytes, stream)
         except Exception as e:
             raise ValueError(f"Error in kernel {self}") from e
 
@@ -139,8 +141,8 @@ class Kernel:
         device = None
         prepared = []
         for args in arg_sets:
-            device, kargs = self._prepare(args)
-            prepared.append(kargs)
+            device = self._prepare(args)
+            prepared.append(list(args))
         spec = self.kernel_spec
         lp = spec.launch_params
         stream = torch.cuda.current_stream(device).cuda_stream

@@ -72,11 +72,18 @@ def test_in_memory_header():
 def test_argument_marshalling_rules():
     """None -> null pointer, int -> 64-bit, float -> 32-bit, more than 16 args rejected
     (reference: spio/cuda/driver.pyx:171-199)."""
-    arr, keep = driver.Function.marshal([None, 5, 2.5])
-    assert isinstance(keep[0], ctypes.c_void_p) and not keep[0].value
-    assert isinstance(keep[1], ctypes.c_longlong) and keep[1].value == 5
-    assert isinstance(keep[2], ctypes.c_float) and keep[2].value == 2.5
-    assert len(arr) == 3
+    params, values = driver.Function.marshal([None, 5, 2.5, -3])
+    assert len(params) == 4
+    # params[i] is the address of the argument's own 8-byte slot, read as the kernel reads it
+    assert ctypes.c_void_p.from_address(params[0]).value is None
+    assert ctypes.c_longlong.from_address(params[1]).value == 5
+    assert ctypes.c_float.from_address(params[2]).value == 2.5
+    assert ctypes.c_longlong.from_address(params[3]).value == -3
+    assert params[1] - params[0] == 8 and params[0] == ctypes.addressof(values)
+    with pytest.raises(ValueError, match="Unsupported"):
+        driver.Function.marshal([True])
+    with pytest.raises(ValueError, match="64-bit"):
+        driver.Function.marshal([1 << 70])
     with pytest.raises(ValueError, match="Too many"):
         driver.Function.marshal([0] * 17)
     with pytest.raises(ValueError, match="Unsupported"):
