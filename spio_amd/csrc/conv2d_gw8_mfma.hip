@@ -129,7 +129,9 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
 
     const int tid = thread_id();
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    // the wave index as a scalar: conditions on it become scalar branches, so that no MFMA
+    // (which ignores the lane mask) is ever issued under an empty mask
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wg = wave % GB;  // group within the workgroup
     const int ws = wave / GB;  // tile split index
 
@@ -175,6 +177,19 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
             }
         }
     }
+    const long long row_units = (long long)SW * kGroups;  // 16-byte units per source row
+    const long long dst_row_units = (long long)DW * kGroups;
+
+    // ---- rows 0..PF-1 into registers, first of all: their latency covers the filter set-up ----
+    spio_uint4 pre[PF][LPT];
+#pragma unroll
+    for (int t = 0; t < PF; ++t) {
+        // rows outside the image are loaded from the nearest real row and never used
+        const int h = imin(imax(p0 + t - EPY, 0), SH - 1);
+#pragma unroll
+        for (int l = 0; l < LPT; ++l) pre[t][l] = load_row(src + in_off[l] + h * row_units, t);
+    }
+
     // ---- loop-invariant addressing of the cooperative row store ----
     int out_off[SPT];  // 16-byte units from dst; row term excluded; -1 = nothing to store
     int out_lds[SPT];  // byte offset inside an output-stage row
@@ -285,18 +300,8 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
     // ---- zero the ring once: halo and slack cells are never written again ----
     for (int i = tid; i < NR * RING_ROW_UNITS; i += THREADS) ring[i] = spio_uint4{0u, 0u, 0u, 0u};
 
-    const long long row_units = (long long)SW * kGroups;  // 16-byte units per source row
-    const long long dst_row_units = (long long)DW * kGroups;
 
-    // ---- prologue: rows 0..PF-1 into registers, row 0 into the ring ----
-    spio_uint4 pre[PF][LPT];
-#pragma unroll
-    for (int t = 0; t < PF; ++t) {
-        // rows outside the image are loaded from the nearest real row and never used
-        const int h = imin(imax(p0 + t - EPY, 0), SH - 1);
-#pragma unroll
-        for (int l = 0; l < LPT; ++l) pre[t][l] = load_row(src + in_off[l] + h * row_units, t);
-    }
+    // ---- row 0 into the ring ----
     block_sync();  // ring zeroed
     {
         const int h = p0 - EPY;

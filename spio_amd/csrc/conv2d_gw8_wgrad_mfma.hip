@@ -54,6 +54,9 @@ using namespace spio;
 #ifndef SPIO_TS
 #define SPIO_TS 1
 #endif
+#ifndef SPIO_RB
+#define SPIO_RB 1
+#endif
 
 namespace {
 
@@ -64,7 +67,8 @@ constexpr int ITERS = SPIO_ITERS;  // image blocks per workgroup
 constexpr int TS = SPIO_TS;        // waves sharing the 32-pixel chunks of one group
 constexpr int WAVES = GB * TS;
 constexpr int THREADS = 64 * WAVES;
-constexpr int PF = SPIO_PF;  // prefetch distance in rows (even)
+constexpr int PF = SPIO_PF;  // prefetch distance in steps (even)
+constexpr int RB = SPIO_RB;  // x rows (and dy rows) per step: 1 or 2
 
 constexpr int S2 = 2 * ((kS + 1) / 2);
 constexpr int NBLK = S2 / 2;   // column-tap pairs
@@ -77,8 +81,10 @@ constexpr int FPX = 32 * KC + S2 - 1;
 constexpr int GSX = FPX + ((9 - FPX % 16) + 16) % 16;  // x group stride (pixels), = 9 mod 16
 constexpr int FPD = 32 * KC;
 constexpr int GSD = FPD + ((9 - FPD % 16) + 16) % 16;  // dy group stride
-constexpr int NRX = 2;                                 // x ring rows
-constexpr int NRD = 2 * ((kR + 2) / 2);                // dy ring rows: even, >= R+1
+constexpr int NRX = 2 * RB;                             // x ring rows: the step's rows and the next step's
+// dy ring rows: the aligned row pairs a step multiplies (R+1 rows with one row per step, up to
+// R+2 with two) plus the rows the step writes for the next one; even.
+constexpr int NRD = 2 * ((kR + 2) / 2) + (RB == 2 ? 2 : 0);
 constexpr int XROW_UNITS = GB * GSX;
 // dy ring rows are 64 bytes apart modulo the 256-byte bank period, so the two rows of a
 // pair that one transposing read touches fall into different banks.
@@ -91,11 +97,24 @@ constexpr int GBLKS = (kGroups + GB - 1) / GB;
 constexpr int PBLKS = (kP + BH - 1) / BH;
 constexpr int NBLKS = (kN + NB * ITERS - 1) / (NB * ITERS);
 constexpr int NUM_BLOCKS = GBLKS * PBLKS * NBLKS;
-constexpr int STEPS = BH + kR - 1;
+constexpr int ROWS = BH + kR - 1;            // x rows a workgroup streams
+constexpr int STEPS = (ROWS + RB - 1) / RB;  // barrier-separated steps of RB rows
+constexpr int NPAIR = kR / 2 + 1;            // aligned dy row pairs one step can touch
+constexpr int CPW = (KC + TS - 1) / TS;      // 32-pixel chunks per wave
 
-static_assert((NRX * XROW_UNITS + NRD * DROW_UNITS) * 16 <= 160 * 1024, "LDS overflow");
+// LDS: the two rings while streaming; at the end the same block holds the reduction scratch:
+// per wave NBLK*128 floats for the row-slot halves, the sums of the other waves of a split
+// group, and (atomic publishing) every group's R*S*64 sums in grad_weight order.
+constexpr int RING_UNITS = NRX * XROW_UNITS + NRD * DROW_UNITS;
+constexpr int SCRATCH_FLOATS = NBLK * 128;  // per wave
+constexpr int RED_FLOATS = GB * (TS - 1) * NBLK * 128;
+constexpr int GROUP_FLOATS = kR * kS * 64;  // grad_weight values of one group
+constexpr int PUBLISH_FLOATS = WAVES * SCRATCH_FLOATS + RED_FLOATS + (SPIO_PARTIALS ? 0 : GB * GROUP_FLOATS);
+constexpr int LDS_UNITS = RING_UNITS > (PUBLISH_FLOATS + 3) / 4 ? RING_UNITS : (PUBLISH_FLOATS + 3) / 4;
+static_assert(LDS_UNITS * 16 <= 160 * 1024, "LDS overflow");
 static_assert(NRD % 2 == 0 && NRD >= kR + 1, "dy ring too small");
 static_assert(PF >= 2 && PF % 2 == 0, "prefetch distance must be even");
+static_assert(RB == 1 || RB == 2, "one or two rows per step");
 constexpr int PART_WAVE_FLOATS = kR * NBLK * 4 * 32;  // floats one wave publishes (partial-block layout)
 
 
@@ -116,13 +135,15 @@ extern "C" __global__ void SPIO_LAUNCH_BOUNDS(THREADS)
 SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__ x,
                  const spio_uint4* __restrict__ dy) {
     // One LDS block: the x ring, then the dy ring; reused as reduction scratch at the end.
-    __shared__ spio_uint4 lds[NRX * XROW_UNITS + NRD * DROW_UNITS];
+    __shared__ spio_uint4 lds[LDS_UNITS];
     spio_uint4* const xring = lds;
     spio_uint4* const dring = lds + NRX * XROW_UNITS;
 
     const int tid = thread_id();
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    // the wave index as a scalar: conditions on it become scalar branches, so that no MFMA
+    // (which ignores the lane mask) is ever issued under an empty mask
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wg = wave % GB;  // group within the workgroup
     const int ws = wave / GB;  // which share of the 32-pixel chunks this wave multiplies
 
@@ -135,10 +156,6 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
     const int bh_eff = imin(BH, kP - p0);  // dy rows that exist in this block
     const int gglob = cb * GB + wg;
     const bool wave_active = gglob < kGroups;
-
-    // zero both rings once: halo, gap and slack cells are never written again
-    for (int i = tid; i < NRX * XROW_UNITS; i += THREADS) xring[i] = spio_uint4{0u, 0u, 0u, 0u};
-    for (int i = tid; i < NRD * DROW_UNITS; i += THREADS) dring[i] = spio_uint4{0u, 0u, 0u, 0u};
 
     // lane roles inside the transposing reads: block kb = lane/16 covers pixels 8*kb..8*kb+7,
     // source lane sigma = lane%16 = 4*jr + t supplies pixel jr (+4 for the second read) of
@@ -164,11 +181,19 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
         if (n0 >= kN) break;
 
         // ---- loop-invariant addressing for this image block ----
+        // Every thread issues the same loads on every step, without branches, so that the
+        // compiler counts outstanding loads exactly and a step waits only for the rows it
+        // needs (a load under a branch makes it wait for all of them, which would serialise the
+        // prefetch).  Cells without data (halo columns, missing images or groups) and rows
+        // outside the tensor load a valid address and become zero when written to LDS.
         int x_off[LPTX], x_lds[LPTX];
+        bool x_ok[LPTX];
+        const int x_dummy = n0 * kH * kW * kGroups;
 #pragma unroll
         for (int l = 0; l < LPTX; ++l) {
             const int cell = tid + THREADS * l;
-            x_off[l] = -1;
+            x_off[l] = x_dummy;
+            x_ok[l] = false;
             x_lds[l] = -1;
             if (cell < X_CELLS) {
                 const int g = cell % GB;
@@ -176,126 +201,186 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
                 const int img = f / WPI;
                 const int col = f % WPI - kPadX;
                 x_lds[l] = g * GSX + f;
-                if (col >= 0 && col < kW && n0 + img < kN && cb * GB + g < kGroups)
+                if (col >= 0 && col < kW && n0 + img < kN && cb * GB + g < kGroups) {
                     x_off[l] = ((n0 + img) * kH * kW + col) * kGroups + cb * GB + g;
+                    x_ok[l] = true;
+                }
             }
         }
         int d_off[LPTD], d_lds[LPTD];
+        bool d_ok[LPTD];
+        const int d_dummy = n0 * kP * kQ * kGroups;
 #pragma unroll
         for (int l = 0; l < LPTD; ++l) {
             const int cell = tid + THREADS * l;
-            d_off[l] = -1;
+            d_off[l] = d_dummy;
+            d_ok[l] = false;
             d_lds[l] = -1;
             if (cell < D_CELLS) {
                 const int g = cell % GB;
                 const int q = (cell / GB) % kQ;
                 const int img = cell / (GB * kQ);
                 d_lds[l] = g * GSD + img * WPI + q;
-                if (n0 + img < kN && cb * GB + g < kGroups)
+                if (n0 + img < kN && cb * GB + g < kGroups) {
                     d_off[l] = ((n0 + img) * kP * kQ + q) * kGroups + cb * GB + g;
+                    d_ok[l] = true;
+                }
             }
         }
+        const spio_uint4 zero4 = spio_uint4{0u, 0u, 0u, 0u};
 
-        // ---- prologue: rows 0..PF-1 into registers, row 0 into LDS ----
-        spio_uint4 xpre[PF][LPTX], dpre[PF][LPTD];
+        // ---- prologue: steps 0..PF-1 into registers, step 0 into LDS ----
+        spio_uint4 xpre[PF][RB][LPTX], dpre[PF][RB][LPTD];
 #pragma unroll
-        for (int t = 0; t < PF; ++t) {
-            const int h = p0 + t - kPadY;
-            const bool x_ok = t < STEPS && h >= 0 && h < kH;
+        for (int sp = 0; sp < PF; ++sp) {
 #pragma unroll
-            for (int l = 0; l < LPTX; ++l) {
-                xpre[t][l] = spio_uint4{0u, 0u, 0u, 0u};
-                if (x_ok && x_off[l] >= 0) xpre[t][l] = load_stream(x + x_off[l] + h * xrow_units);
+            for (int rr = 0; rr < RB; ++rr) {
+                const int t = sp * RB + rr;
+                const int h = imin(imax(p0 + t - kPadY, 0), kH - 1);
+#pragma unroll
+                for (int l = 0; l < LPTX; ++l) xpre[sp][rr][l] = load_stream(x + x_off[l] + h * xrow_units);
+                const int pr = imin(p0 + t, kP - 1);
+#pragma unroll
+                for (int l = 0; l < LPTD; ++l) dpre[sp][rr][l] = load_stream(dy + d_off[l] + pr * drow_units);
             }
-            const bool d_ok = t < bh_eff;
-#pragma unroll
-            for (int l = 0; l < LPTD; ++l) {
-                dpre[t][l] = spio_uint4{0u, 0u, 0u, 0u};
-                if (d_ok && d_off[l] >= 0) dpre[t][l] = load_stream(dy + d_off[l] + (p0 + t) * drow_units);
-            }
+        }
+        if (it == 0) {
+            // zero both rings once, while the first loads are in flight: halo, gap and slack
+            // cells are never written again
+            for (int i = tid; i < NRX * XROW_UNITS; i += THREADS) xring[i] = zero4;
+            for (int i = tid; i < NRD * DROW_UNITS; i += THREADS) dring[i] = zero4;
         }
         block_sync();  // rings zeroed / previous image block finished
 #pragma unroll
-        for (int l = 0; l < LPTX; ++l)
-            if (x_lds[l] >= 0) xring[x_lds[l]] = xpre[0][l];
+        for (int rr = 0; rr < RB; ++rr) {
+            const int h = p0 + rr - kPadY;
+            const bool xrow_ok = h >= 0 && h < kH;
 #pragma unroll
-        for (int l = 0; l < LPTD; ++l)
-            if (d_lds[l] >= 0) dring[d_lds[l]] = dpre[0][l];
+            for (int l = 0; l < LPTX; ++l)
+                if (x_lds[l] >= 0) xring[rr * XROW_UNITS + x_lds[l]] = (xrow_ok && x_ok[l]) ? xpre[0][rr][l] : zero4;
+            const bool drow_ok = rr < bh_eff;
+#pragma unroll
+            for (int l = 0; l < LPTD; ++l)
+                if (d_lds[l] >= 0) dring[rr * DROW_UNITS + d_lds[l]] = (drow_ok && d_ok[l]) ? dpre[0][rr][l] : zero4;
+        }
         block_sync();
 
-        for (int tb = 0; tb < STEPS; tb += PF) {
+        for (int sb = 0; sb < STEPS; sb += PF) {
 #pragma unroll
             for (int uf = 0; uf < PF; ++uf) {
-                const int t = tb + uf;
-                if (t >= STEPS) break;
-                const int uu = uf & 1;  // parity of t: x ring row and the parity of delta
+                const int st = sb + uf;
+                if (st >= STEPS) break;
+                const int t = st * RB;  // first x row of the step, relative to the block
+                // PF is even, so the parity of the step is known at compile time: it fixes the
+                // x ring rows and, with one row per step, the parity of delta.
+                const int sp = uf & 1;
 
-                // 1. prefetch rows t+PF (their register buffer held row t, now in LDS)
-                {
-                    const int t2 = t + PF;
-                    const int h = p0 + t2 - kPadY;
-                    const bool x_ok = t2 < STEPS && h >= 0 && h < kH;
+                // 1. read this step's fragments: the x rows t+rr and the aligned dy row pairs
+                //    they overlap (x row t+rr and the pair starting at row i2 meet at
+                //    delta = t + rr - i2).  All LDS reads are issued before anything else so that
+                //    their latency, the global loads and the ring writes below overlap; the
+                //    MFMAs come last.
+                const int tbase = RB == 2 ? t : t - sp;  // even
+                bool row_live[RB];
+                bool any_live = false;
 #pragma unroll
-                    for (int l = 0; l < LPTX; ++l) {
-                        spio_uint4 v = spio_uint4{0u, 0u, 0u, 0u};
-                        if (x_ok && x_off[l] >= 0) v = load_stream(x + x_off[l] + h * xrow_units);
-                        xpre[uf][l] = v;
-                    }
-                    const bool d_ok = t2 < bh_eff;
-#pragma unroll
-                    for (int l = 0; l < LPTD; ++l) {
-                        spio_uint4 v = spio_uint4{0u, 0u, 0u, 0u};
-                        if (d_ok && d_off[l] >= 0) v = load_stream(dy + d_off[l] + (p0 + t2) * drow_units);
-                        dpre[uf][l] = v;
-                    }
+                for (int rr = 0; rr < RB; ++rr) {
+                    const int hcur = p0 + t + rr - kPadY;
+                    row_live[rr] = t + rr < ROWS && hcur >= 0 && hcur < kH;
+                    any_live = any_live || row_live[rr];
                 }
-
-                // 2. x row t against the dy row pairs it overlaps
-                const int hcur = p0 + t - kPadY;
-                if (wave_active && hcur >= 0 && hcur < kH) {
-                    const unsigned char* xrow =
-                        reinterpret_cast<const unsigned char*>(xring + uu * XROW_UNITS) + xfrag_off;
+                const bool do_math = wave_active && any_live;
+                spio_half8 bfrag[CPW][RB][NBLK], afrag[CPW][NPAIR];
+                if (do_math) {
 #pragma unroll
-                    for (int ci = 0; ci < (KC + TS - 1) / TS; ++ci) {
+                    for (int ci = 0; ci < CPW; ++ci) {
                         const int ch = ws + TS * ci;
                         if (TS > 1 && ch >= KC) break;
-                        spio_half8 bfrag[NBLK];
 #pragma unroll
-                        for (int nb = 0; nb < NBLK; ++nb) {
-                            const unsigned char* pb0 = xrow + (32 * ch + 2 * nb) * 16;
-                            bfrag[nb] = read_tr_pair(pb0, pb0 + 4 * 16);
+                        for (int rr = 0; rr < RB; ++rr) {
+                            const unsigned char* xrow =
+                                reinterpret_cast<const unsigned char*>(xring + (sp * RB + rr) * XROW_UNITS) + xfrag_off;
+#pragma unroll
+                            for (int nb = 0; nb < NBLK; ++nb) {
+                                const unsigned char* pb0 = xrow + (32 * ch + 2 * nb) * 16;
+                                bfrag[ci][rr][nb] = read_tr_pair(pb0, pb0 + 4 * 16);
+                            }
                         }
 #pragma unroll
-                        for (int d = uu; d < ND; d += 2) {
-                            // delta = d has the parity of t: pair index i = (t - d) / 2
-                            const int i2 = t - d;  // first row of the pair, relative to p0
+                        for (int m = 0; m < NPAIR; ++m) {
+                            const int i2 = tbase - 2 * m;  // first row of the pair, relative to p0
                             if (i2 >= 0 && i2 < bh_eff) {
                                 const int slot = (i2 + sel) % NRD;
                                 const unsigned char* pa0 =
                                     reinterpret_cast<const unsigned char*>(dring + slot * DROW_UNITS) +
                                     dfrag_off + (32 * ch) * 16;
-                                const spio_half8 afrag = read_tr_pair(pa0, pa0 + 4 * 16);
-#pragma unroll
-                                for (int nb = 0; nb < NBLK; ++nb)
-                                    acc[d][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                                        afrag, bfrag[nb], acc[d][nb], 0, 0, 0);
+                                afrag[ci][m] = read_tr_pair(pa0, pa0 + 4 * 16);
                             }
                         }
                     }
                 }
 
-                // 3. rows t+1 into LDS
-                if (t + 1 < STEPS) {
-                    const int hn = p0 + t + 1 - kPadY;
-                    if (hn >= 0 && hn < kH) {
+                // 2. prefetch step st+PF (its register buffer held step st, now in LDS); rows
+                //    past the end repeat a real row and are never used
 #pragma unroll
-                        for (int l = 0; l < LPTX; ++l)
-                            if (x_lds[l] >= 0) xring[((uu + 1) & 1) * XROW_UNITS + x_lds[l]] = xpre[(uf + 1) % PF][l];
+                for (int rr = 0; rr < RB; ++rr) {
+                    const int t2 = (st + PF) * RB + rr;
+                    const int h = imin(imax(p0 + t2 - kPadY, 0), kH - 1);
+#pragma unroll
+                    for (int l = 0; l < LPTX; ++l) xpre[uf][rr][l] = load_stream(x + x_off[l] + h * xrow_units);
+                    const int pr = imin(p0 + t2, kP - 1);
+#pragma unroll
+                    for (int l = 0; l < LPTD; ++l) dpre[uf][rr][l] = load_stream(dy + d_off[l] + pr * drow_units);
+                }
+
+                // 3. the rows of step st+1 into LDS (dy rows past the block's last row become
+                //    zero).  The ring rows written here are not read in this step, except for dy
+                //    entries whose filter row is out of range and whose product is ignored.
+                if (st + 1 < STEPS) {
+#pragma unroll
+                    for (int rr = 0; rr < RB; ++rr) {
+                        const int tn = t + RB + rr;
+                        const int hn = p0 + tn - kPadY;
+                        if (tn < ROWS && hn >= 0 && hn < kH) {
+#pragma unroll
+                            for (int l = 0; l < LPTX; ++l)
+                                if (x_lds[l] >= 0)
+                                    xring[(((sp + 1) & 1) * RB + rr) * XROW_UNITS + x_lds[l]] =
+                                        x_ok[l] ? xpre[(uf + 1) % PF][rr][l] : zero4;
+                        }
+                        const int dslot = tn % NRD;
+                        const bool drow_ok = tn < bh_eff;
+#pragma unroll
+                        for (int l = 0; l < LPTD; ++l)
+                            if (d_lds[l] >= 0)
+                                dring[dslot * DROW_UNITS + d_lds[l]] =
+                                    (drow_ok && d_ok[l]) ? dpre[(uf + 1) % PF][rr][l] : zero4;
                     }
-                    const int dslot = (t + 1) % NRD;
+                }
+
+                // 4. multiply
+                if (do_math) {
 #pragma unroll
-                    for (int l = 0; l < LPTD; ++l)
-                        if (d_lds[l] >= 0) dring[dslot * DROW_UNITS + d_lds[l]] = dpre[(uf + 1) % PF][l];
+                    for (int ci = 0; ci < CPW; ++ci) {
+                        const int ch = ws + TS * ci;
+                        if (TS > 1 && ch >= KC) break;
+#pragma unroll
+                        for (int m = 0; m < NPAIR; ++m) {
+                            const int i2 = tbase - 2 * m;
+                            if (i2 >= 0 && i2 < bh_eff) {
+#pragma unroll
+                                for (int rr = 0; rr < RB; ++rr) {
+                                    const int d = (RB == 2 ? rr : sp) + 2 * m;  // = t + rr - i2
+                                    if (d <= kR && row_live[rr]) {
+#pragma unroll
+                                        for (int nb = 0; nb < NBLK; ++nb)
+                                            acc[d][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                                afrag[ci][m], bfrag[ci][rr][nb], acc[d][nb], 0, 0, 0);
+                                    }
+                                }
+                            }
+                        }
+                    }
                 }
                 block_sync();
             }
@@ -309,13 +394,13 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
     // one group then add their sums through LDS so that only one wave per group publishes:
     // fp32 atomics into grad_weight, or plain stores into this workgroup's partial image when a
     // second kernel does the reduction.
-    constexpr int SCRATCH_FLOATS = NBLK * 128;  // per wave
-    static_assert((WAVES * SCRATCH_FLOATS + GB * (TS - 1) * NBLK * 128) * 4 <= (NRX * XROW_UNITS + NRD * DROW_UNITS) * 16,
-                  "reduction scratch does not fit in LDS");
     block_sync();  // every wave is done with the rings; reuse them as scratch
     {
         float* scratch = reinterpret_cast<float*>(lds) + wave * SCRATCH_FLOATS;
         float* red = reinterpret_cast<float*>(lds) + WAVES * SCRATCH_FLOATS;  // [group][ts-1][nb][e][32 lanes]
+        // this group's sums in grad_weight order [k][r][s][c] (atomic publishing only)
+        float* gstage = reinterpret_cast<float*>(lds) + WAVES * SCRATCH_FLOATS + RED_FLOATS + wg * GROUP_FLOATS;
+        (void)gstage;
         const int k4 = 4 * ((lane >> 4) & 1);
         const int sj = (lane & 15) >> 3;
         const int c = lane & 7;
@@ -383,14 +468,24 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
                     if (s < kS) {
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
-                            atomic_add_f32(out + (((long long)(8 * gglob + k4 + e) * kR + r) * kS + s) * 8 + c,
-                                           total[nb][e]);
+                            gstage[(((k4 + e) * kR + r) * kS + s) * 8 + c] = total[nb][e];
                     }
                 }
             }
 #endif
             if (TS > 1) block_sync();  // the scratch is rewritten for the next filter row
         }
+#if !SPIO_PARTIALS
+        // One wave per group adds the group's R*S*64 sums into grad_weight: every atomic
+        // instruction covers 64 consecutive floats (two full 128-byte lines), which the memory
+        // system retires several times faster than the scattered half-lines of the accumulator
+        // layout.  The wave reads back what it wrote itself, so no barrier is needed.
+        if (wave_active && ws == 0) {
+            float* gout = out + (long long)gglob * GROUP_FLOATS;
+#pragma unroll
+            for (int i = 0; i < kR * kS; ++i) atomic_add_f32(gout + 64 * i + lane, gstage[64 * i + lane]);
+        }
+#endif
     }
 
 }

@@ -5,7 +5,7 @@ its partial sums into a pre-zeroed fp32 tensor laid out [K][R][S][8]
 (spio/functional/conv2d_gw8_function.py:124-130).
 """
 
-from dataclasses import dataclass
+from dataclasses import dataclass, replace
 from typing import Dict, List
 
 import torch
@@ -25,7 +25,8 @@ MAX_WAVES = 16
 MAX_LDS_BYTES = 128 * 1024
 MAX_LOADS_PER_THREAD = 8
 MAX_ACCUMULATORS = 32
-MAX_CONFIGS = 32
+MAX_GEOMETRIES = 12
+PIPELINE_CHOICES = ((2, 1), (4, 1), (2, 2))  # (prefetch, rows)
 
 
 @dataclass(frozen=True)
@@ -38,7 +39,10 @@ class Conv2dGw8WgradConfig:
         block_n: images whose rows are laid side by side in one staged row.
         block_n_iters: image blocks a workgroup accumulates before its atomics.
         chunks: (direct variant only) pixel chunks per group.
-        prefetch: rows of global loads in flight ahead of the computed row (even).
+        prefetch: steps of global loads in flight ahead of the computed step (even).
+        rows: rows of x (and of grad_output) a workgroup multiplies between two barriers,
+            1 or 2; two rows share their grad_output fragments and halve the barriers at the
+            price of a deeper LDS ring.
         split: waves sharing the 32-pixel chunks of one group; their sums are added in LDS
             before publishing, so bigger workgroups do not publish more.
         two_stage: 1 = workgroups store partial sums to a workspace and a second kernel
@@ -55,6 +59,7 @@ class Conv2dGw8WgradConfig:
     prefetch: int = 2
     two_stage: int = 0
     split: int = 1
+    rows: int = 1
 
 
 def wgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig) -> Dict[str, int]:
@@ -70,16 +75,21 @@ def wgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig) -> Dic
     gsx = fpx + ((9 - fpx % 16) + 16) % 16
     fpd = 32 * kc
     gsd = fpd + ((9 - fpd % 16) + 16) % 16
-    nrd = 2 * ((r + 2) // 2)
+    rb = config.rows
+    nrx = 2 * rb
+    nrd = 2 * ((r + 2) // 2) + (2 if rb == 2 else 0)
     threads = 64 * gb * ts
-    lds_rings = (2 * gb * gsx + nrd * (gb * gsd + ((4 - (gb * gsd) % 16) + 16) % 16)) * 16
-    lds_scratch = (gb * ts * (s2 // 2) * 128 + gb * (ts - 1) * (s2 // 2) * 128) * 4
+    lds_rings = (nrx * gb * gsx + nrd * (gb * gsd + ((4 - (gb * gsd) % 16) + 16) % 16)) * 16
+    # the same LDS block holds the reduction scratch at the end: per-wave row-slot halves, the
+    # sums of the other waves of a split group, and (atomic publishing) every group's R*S*64 sums
+    lds_scratch = (gb * ts * (s2 // 2) * 128 + gb * (ts - 1) * (s2 // 2) * 128
+                   + (0 if config.two_stage else gb * r * s * 64)) * 4  # fmt: skip
     g = dict(
         NBLK=s2 // 2, ND=r + 1, WPI=wpi, F=f, KC=kc, GSX=gsx, GSD=gsd, NRD=nrd, THREADS=threads,
-        LDS_BYTES=lds_rings, SCRATCH_BYTES=lds_scratch,
+        LDS_BYTES=max(lds_rings, lds_scratch), RING_BYTES=lds_rings, SCRATCH_BYTES=lds_scratch,
         LPTX=divup(f * gb, threads), LPTD=divup(nb * params.q * gb, threads),
         GBLKS=divup(params.groups, gb), PBLKS=divup(params.p, bh),
-        NBLKS=divup(params.n, nb * iters), STEPS=bh + r - 1,
+        NBLKS=divup(params.n, nb * iters), STEPS=divup(bh + r - 1, rb),
         PIXEL_EFF=kspan and (nb * params.q) / (32.0 * kc),
     )  # fmt: skip
     g["NUM_BLOCKS"] = g["GBLKS"] * g["PBLKS"] * g["NBLKS"]
@@ -91,7 +101,6 @@ def _mfma_config_is_legal(params, config) -> bool:
     return (
         config.groups * config.split <= MAX_WAVES
         and config.split <= g["KC"]
-        and g["SCRATCH_BYTES"] <= g["LDS_BYTES"]
         and config.block_h <= params.p
         and config.block_n * config.block_n_iters <= max(params.n, 1)
         and g["LDS_BYTES"] <= MAX_LDS_BYTES
@@ -99,7 +108,8 @@ def _mfma_config_is_legal(params, config) -> bool:
         and g["ND"] * g["NBLK"] <= MAX_ACCUMULATORS
         and config.prefetch >= 2
         and config.prefetch % 2 == 0
-        and (g["LPTX"] + g["LPTD"]) * config.prefetch <= 32
+        and config.rows in (1, 2)
+        and (g["LPTX"] + g["LPTD"]) * config.prefetch * config.rows <= 32
     )
 
 
@@ -109,7 +119,6 @@ def _mfma_score(params, config, num_cus) -> float:
     halo = (config.block_h + params.r - 1) / config.block_h
     traffic = 1.0 + 0.5 * (halo - 1.0)
     group_eff = params.groups / (g["GBLKS"] * config.groups)
-    per_cu = max(1, min(160 * 1024 // g["LDS_BYTES"], 2048 // g["THREADS"], 8))
     # compute units idle in the last round of workgroups
     quant = divup(g["NUM_BLOCKS"], num_cus) * num_cus / g["NUM_BLOCKS"]
     # Publishing costs R*S*64 values per (workgroup, group): atomics retire at roughly 128 per
@@ -121,9 +130,8 @@ def _mfma_score(params, config, num_cus) -> float:
         publish_us = 4.5 + 2.0 * 4.0 * values / 5.0e6
     else:
         publish_us = values / (128 * 2.1e3)
-    few_waves = 1.15 if min(per_cu, max(1, g["NUM_BLOCKS"] // num_cus)) * g["THREADS"] < 512 else 1.0
     split_line = 1.0 if (config.groups * 16) % 128 == 0 or config.groups == params.groups else 1.12
-    return (traffic * quant * few_waves * split_line / (g["PIXEL_EFF"] ** 0.3 * group_eff)) * (
+    return (traffic * quant * split_line / (g["PIXEL_EFF"] ** 0.3 * group_eff)) * (
         1.0 + publish_us / stream_us
     )
 
@@ -134,23 +142,28 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None) -> List[Conv2dGw8Wgr
     G = params.groups
     group_choices = sorted({g for g in (4, 8, 16, G) if g <= min(G, MAX_WAVES)}) or [min(G, MAX_WAVES)]
     row_choices = sorted({bh for bh in (4, 7, 8, 14, 16, 28, 32, 56, params.p) if bh <= params.p})
-    found = []
+    # Rank the tile geometries first and keep the best few; each of them is then tried with the
+    # pipeline variants (prefetch distance, rows per step), which the score cannot tell apart.
+    geometries = []
     for gb in group_choices:
         for nb in (1, 2, 4, 8):
             for iters in (1, 2, 4, 8):
                 for bh in row_choices:
-                    for pf in (2, 4, 8):
-                        if pf > 2 and pf > bh + params.r - 1:
-                            continue
-                        for two_stage in (0, 1):
-                            for ts in (1, 2):
-                                cfg = Conv2dGw8WgradConfig(groups=gb, block_h=bh, block_n=nb,
-                                                           block_n_iters=iters, prefetch=pf,
-                                                           two_stage=two_stage, split=ts)  # fmt: skip
-                                if _mfma_config_is_legal(params, cfg):
-                                    found.append((_mfma_score(params, cfg, num_cus), cfg))
-    found.sort(key=lambda sc: sc[0])
-    configs = [cfg for _, cfg in found[:MAX_CONFIGS]]
+                    for two_stage in (0, 1):
+                        for ts in (1, 2):
+                            cfg = Conv2dGw8WgradConfig(groups=gb, block_h=bh, block_n=nb, block_n_iters=iters,
+                                                       prefetch=2, two_stage=two_stage, split=ts)  # fmt: skip
+                            if _mfma_config_is_legal(params, cfg):
+                                geometries.append((_mfma_score(params, cfg, num_cus), cfg))
+    geometries.sort(key=lambda sc: sc[0])
+    configs = []
+    for _, base in geometries[:MAX_GEOMETRIES]:
+        for pf, rows in PIPELINE_CHOICES:
+            if pf > 2 and pf * rows > base.block_h + params.r - 1:
+                continue
+            cfg = replace(base, prefetch=pf, rows=rows)
+            if _mfma_config_is_legal(params, cfg):
+                configs.append(cfg)
     total_pix = params.n * params.p * params.q
     chunks = max(1, min(divup(8 * num_cus, params.groups), divup(total_pix, 64)))
     configs.append(Conv2dGw8WgradConfig(groups=1, block_h=1, block_n=1, block_n_iters=1,
@@ -173,7 +186,7 @@ def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig, _dev
     g = wgrad_geometry(params, config)
     defines.update(SPIO_GB=config.groups, SPIO_BH=config.block_h, SPIO_NB=config.block_n,
                    SPIO_ITERS=config.block_n_iters, SPIO_PF=config.prefetch,
-                   SPIO_TS=config.split)  # fmt: skip
+                   SPIO_TS=config.split, SPIO_RB=config.rows)  # fmt: skip
     spec = KernelSpec(defines, LaunchParams(grid=g["NUM_BLOCKS"], block=g["THREADS"]), MFMA_SOURCE, notes=g)
     if config.two_stage:
         num_partials = g["NBLKS"] * g["PBLKS"]
