@@ -109,7 +109,11 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
 // zero (or hold a value to accumulate onto) before the launch.
 extern "C" __global__ void SPIO_LAUNCH_BOUNDS(SPIO_BLOCK_THREADS)
 SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_half* __restrict__ x,
-                 const spio_half* __restrict__ dy) {
+                 const spio_half* __restrict__ dy
+#if SPIO_HAS_BIAS
+                 , float* __restrict__ grad_bias  // [K] fp32, accumulated into; null = not wanted
+#endif
+) {
     constexpr int kWaves = SPIO_BLOCK_THREADS / 64;
     const int g = block_id() % kGroups;
     const int chunk = block_id() / kGroups;
@@ -128,12 +132,14 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_half* __restrict__ 
 #pragma unroll
     for (int t = 0; t < kR * kS; ++t) acc[t] = 0.f;
 
+    float dsum = 0.f;  // grad_output summed over this wave's pixels (same in the 8 lanes of a k)
     for (long long pix = begin + wave; pix < end; pix += kWaves) {
         const int q = (int)(pix % kQ);
         const long long t0 = pix / kQ;
         const int p = (int)(t0 % kP);
         const int n = (int)(t0 / kP);
         const float d = (float)dy[pix * kC + 8 * g + k];
+        dsum += d;
 #pragma unroll
         for (int r = 0; r < kR; ++r) {
             const int ih = p + r - kPadY;
@@ -153,6 +159,11 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_half* __restrict__ 
         for (int s = 0; s < kS; ++s)
             atomic_add_f32(grad_weight + ((((long long)(8 * g + k)) * kR + r) * kS + s) * 8 + c,
                       acc[r * kS + s]);
+#if SPIO_HAS_BIAS
+    if (grad_bias != nullptr && c == 0) atomic_add_f32(grad_bias + 8 * g + k, dsum);
+#else
+    (void)dsum;
+#endif
 }
 
 #endif  // SPIO_WGRAD

@@ -57,6 +57,9 @@ using namespace spio;
 #ifndef SPIO_RB
 #define SPIO_RB 1
 #endif
+#ifndef SPIO_HAS_BIAS
+#define SPIO_HAS_BIAS 0
+#endif
 
 namespace {
 
@@ -97,7 +100,10 @@ constexpr int GBLKS = (kGroups + GB - 1) / GB;
 constexpr int PBLKS = (kP + BH - 1) / BH;
 constexpr int NBLKS = (kN + NB * ITERS - 1) / (NB * ITERS);
 constexpr int NUM_BLOCKS = GBLKS * PBLKS * NBLKS;
-constexpr int ROWS = BH + kR - 1;            // x rows a workgroup streams
+constexpr bool kDbias = SPIO_HAS_BIAS != 0;  // also sum grad_output per channel (grad_bias)
+// x rows a workgroup streams.  The bias sum takes a grad_output row pair one step after its
+// first row was staged, so a one-row filter needs one more step when the sum is wanted.
+constexpr int ROWS = BH + (kDbias && kR == 1 ? 2 : kR) - 1;
 constexpr int STEPS = (ROWS + RB - 1) / RB;  // barrier-separated steps of RB rows
 constexpr int NPAIR = kR / 2 + 1;            // aligned dy row pairs one step can touch
 constexpr int CPW = (KC + TS - 1) / TS;      // 32-pixel chunks per wave
@@ -133,7 +139,11 @@ SPIO_DEVICE spio_half8 read_tr_pair(const unsigned char* lo, const unsigned char
 
 extern "C" __global__ void SPIO_LAUNCH_BOUNDS(THREADS)
 SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__ x,
-                 const spio_uint4* __restrict__ dy) {
+                 const spio_uint4* __restrict__ dy
+#if SPIO_HAS_BIAS
+                 , float* __restrict__ grad_bias  // [K] fp32, accumulated into; null = not wanted
+#endif
+) {
     // One LDS block: the x ring, then the dy ring; reused as reduction scratch at the end.
     __shared__ spio_uint4 lds[LDS_UNITS];
     spio_uint4* const xring = lds;
@@ -173,6 +183,11 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
 #pragma unroll
         for (int nb = 0; nb < NBLK; ++nb) acc[d][nb] = spio_float4{0.f, 0.f, 0.f, 0.f};
 
+    // grad_bias rides along as one more MFMA per chunk and row pair: dy (A) times an all-ones B
+    // gives, in every column, the sum of the 32 pixels for the 16 (row slot, channel) rows.
+    spio_float4 accb = spio_float4{0.f, 0.f, 0.f, 0.f};
+    const spio_half8 ones8 = spio_half8{1, 1, 1, 1, 1, 1, 1, 1};
+    (void)ones8;
     const long long xrow_units = (long long)kW * kGroups;
     const long long drow_units = (long long)kQ * kGroups;
 
@@ -289,7 +304,11 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
                     row_live[rr] = t + rr < ROWS && hcur >= 0 && hcur < kH;
                     any_live = any_live || row_live[rr];
                 }
-                const bool do_math = wave_active && any_live;
+                // The row pair starting at tbase is complete in LDS (its second row was staged
+                // during the previous step) when two rows go per step, and on odd steps otherwise;
+                // that is when it is added to the bias sum, once per pair.
+                const bool bias_pair = kDbias && (RB == 2 || sp == 1) && tbase < bh_eff;
+                const bool do_math = wave_active && (any_live || bias_pair);
                 spio_half8 bfrag[CPW][RB][NBLK], afrag[CPW][NPAIR];
                 if (do_math) {
 #pragma unroll
@@ -378,6 +397,8 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
                                                 afrag[ci][m], bfrag[ci][rr][nb], acc[d][nb], 0, 0, 0);
                                     }
                                 }
+                                if (m == 0 && bias_pair)
+                                    accb = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[ci][0], ones8, accb, 0, 0, 0);
                             }
                         }
                     }
@@ -475,6 +496,26 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
 #endif
             if (TS > 1) block_sync();  // the scratch is rewritten for the next filter row
         }
+#if SPIO_HAS_BIAS
+        // grad_bias[8g + k] = accb of row slot 0 (lanes 0-31) + row slot 1 (lanes 32-63); every
+        // column holds the same sum, lanes 0 and 16 publish channels 0-3 and 4-7.
+        {
+            if (lane >= 32) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) scratch[e * 32 + (lane - 32)] = accb[e];
+            }
+            float tb[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                tb[e] = 0.f;
+                if (lane < 32) tb[e] = accb[e] + scratch[e * 32 + lane];
+            }
+            if (wave_active && grad_bias != nullptr && (lane & 47) == 0) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) atomic_add_f32(grad_bias + 8 * gglob + k4 + e, tb[e]);
+            }
+        }
+#endif
 #if !SPIO_PARTIALS
         // One wave per group adds the group's R*S*64 sums into grad_weight: every atomic
         // instruction covers 64 consecutive floats (two full 128-byte lines), which the memory

@@ -132,18 +132,24 @@ def conv2d_gw8_backward_op(
     params = Conv2dGw8Params.from_tensors(inputs, weight, bias, padding=(padding_y, padding_x))
     assert tuple(grad_output.shape) == params.output_shape
 
+    grad_bias = None
     if needs_weight_grad:
         # The kernel accumulates into grad_weight, so it starts from zero; fp32.
         grad_weight = torch.zeros_like(weight, dtype=torch.float32)
         kernel = conv2d_gw8_wgrad_kernel_factory.get_kernel(params, inputs.device)
-        kernel(grad_weight, inputs, grad_output)
+        if params.has_bias:
+            # With a bias the weight-gradient kernel also sums grad_output per channel while it
+            # streams it (the reference runs a separate reduction, conv2d_gw8_function.py:134-136).
+            if needs_bias_grad:
+                grad_bias = torch.zeros(params.c, dtype=torch.float32, device=inputs.device)
+            kernel(grad_weight, inputs, grad_output, grad_bias)
+        else:
+            kernel(grad_weight, inputs, grad_output)
     else:
         grad_weight = None
 
-    if needs_bias_grad:
+    if needs_bias_grad and grad_bias is None:
         grad_bias = grad_output.sum(dim=(0, 2, 3), dtype=torch.float32)
-    else:
-        grad_bias = None
 
     if needs_input_grad:
         grad_input = torch.empty_like(inputs)

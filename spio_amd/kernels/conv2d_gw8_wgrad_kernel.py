@@ -1,5 +1,10 @@
 """Weight-gradient kernel family of conv2d_gw8.
 
+Kernel arguments: (grad_weight, x, grad_output) and, when the params have a
+bias, a fourth `grad_bias` ([K] fp32, pre-zeroed like grad_weight, or None):
+the kernels then also sum grad_output per channel in the same pass, which the
+reference leaves to a separate reduction (spio/functional/conv2d_gw8_function.py:134-136).
+
 Reference: spio/kernels/conv2d_gw8_wgrad_kernel.py:27-285.  The kernel adds
 its partial sums into a pre-zeroed fp32 tensor laid out [K][R][S][8]
 (spio/functional/conv2d_gw8_function.py:124-130).
@@ -89,7 +94,8 @@ def wgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig) -> Dic
         LDS_BYTES=max(lds_rings, lds_scratch), RING_BYTES=lds_rings, SCRATCH_BYTES=lds_scratch,
         LPTX=divup(f * gb, threads), LPTD=divup(nb * params.q * gb, threads),
         GBLKS=divup(params.groups, gb), PBLKS=divup(params.p, bh),
-        NBLKS=divup(params.n, nb * iters), STEPS=divup(bh + r - 1, rb),
+        NBLKS=divup(params.n, nb * iters),
+        STEPS=divup(bh + (2 if params.has_bias and r == 1 else r) - 1, rb),
         PIXEL_EFF=kspan and (nb * params.q) / (32.0 * kc),
     )  # fmt: skip
     g["NUM_BLOCKS"] = g["GBLKS"] * g["PBLKS"] * g["NBLKS"]
@@ -174,6 +180,8 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None) -> List[Conv2dGw8Wgr
 def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig, _device_attr=None) -> KernelSpec:
     params.validate()
     defines = _shape_defines(params)
+    # with a bias the kernels take a fourth pointer and also accumulate grad_bias
+    defines["SPIO_HAS_BIAS"] = int(params.has_bias)
     if config.variant == "direct":
         threads = 256
         defines.update(SPIO_WGRAD=1, SPIO_BLOCK_THREADS=threads, SPIO_WGRAD_CHUNKS=config.chunks)
@@ -202,11 +210,13 @@ def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig, _dev
 
 
 def _make_test_args(params: Conv2dGw8Params, device):
-    """Synthetic (grad_weight, x, dy) for timing."""
+    """Synthetic (grad_weight, x, dy[, grad_bias]) for timing."""
     cl = torch.channels_last
     x = torch.randn(params.input_shape, device=device, dtype=torch.float16).contiguous(memory_format=cl)
     dy = torch.randn(params.output_shape, device=device, dtype=torch.float16).contiguous(memory_format=cl)
     dw = torch.zeros(params.weight_shape, device=device, dtype=torch.float32).contiguous(memory_format=cl)
+    if params.has_bias:
+        return (dw, x, dy, torch.zeros(params.c, device=device, dtype=torch.float32))
     return (dw, x, dy)
 
 

@@ -155,7 +155,15 @@ def run_grad_kernel_test(factory, params: Conv2dGw8Params, configs=None, seed=0,
             out = torch.zeros(params.weight_shape, device="cuda", dtype=torch.float32).contiguous(
                 memory_format=torch.channels_last
             )
-            kernel(out, xg, dyg)
-            torch.cuda.synchronize()
+            if params.has_bias:
+                # with a bias the kernel also sums grad_output per channel into its fourth argument
+                db = torch.zeros(params.c, device="cuda", dtype=torch.float32)
+                kernel(out, xg, dyg, db)
+                torch.cuda.synchronize()
+                oracle.check_close(db, _db_e, acc_depth=params.n * params.p * params.q,
+                                   what=f"grad_bias {params.encode()} {kernel.config}")  # fmt: skip
+            else:
+                kernel(out, xg, dyg)
+                torch.cuda.synchronize()
             oracle.check_close(out, dw_e, acc_depth=depth, what=f"wgrad {params.encode()} {kernel.config}")
         kernel.unload()

@@ -94,8 +94,18 @@ def test_backward_op_skips_what_is_not_needed():
     args = (to_gpu(x), to_gpu(w), to_gpu(b), to_gpu(dy), 1, 1)
     dx, dw, db = torch.ops.spio.conv2d_gw8_backward(*args, False, True, False)
     assert dx is None and db is None and dw.dtype == torch.float32 and dw.shape == w.shape
+    _dx_e, dw_e, db_e = oracle.grads_torch(x, w, b, dy, 1, 1)
+    # weight gradient without bias gradient: the fused kernel gets a null grad_bias pointer
+    oracle.check_close(dw, dw_e, acc_depth=2 * 8 * 8, what="dw only")
     dx, dw, db = torch.ops.spio.conv2d_gw8_backward(*args, True, False, True)
     assert dw is None and dx.dtype == torch.float16 and db.dtype == torch.float32
+    # bias gradient without weight gradient: the separate reduction
+    oracle.check_close(db, db_e, acc_depth=2 * 8 * 8, what="db only")
+    # both: grad_bias comes out of the weight-gradient kernel's own pass over grad_output
+    dx, dw, db = torch.ops.spio.conv2d_gw8_backward(*args, False, True, True)
+    assert dx is None
+    oracle.check_close(dw, dw_e, acc_depth=2 * 8 * 8, what="dw fused")
+    oracle.check_close(db, db_e, acc_depth=2 * 8 * 8, what="db fused")
     # only the input requires grad
     xg = to_gpu(x).requires_grad_(True)
     y = _call(p, xg, to_gpu(w), to_gpu(b))

@@ -29,6 +29,10 @@ SANITY = [
     Conv2dGw8Params(n=2, c=40, h=9, w=9, r=5, s=5, padding=2, has_bias=True),
     Conv2dGw8Params(n=2, c=32, h=14, w=14, r=7, s=7, padding=3, has_bias=False),
     Conv2dGw8Params(n=5, c=8, h=7, w=7, r=2, s=5, padding=(1, 2), has_bias=True),
+    # one filter row with a bias and an odd row count: the fused bias sum needs its extra step
+    Conv2dGw8Params(n=3, c=16, h=9, w=11, r=1, s=3, padding=(0, 1), has_bias=True),
+    # output taller than the input, with a bias: grad_output rows whose x row is all padding
+    Conv2dGw8Params(n=2, c=16, h=6, w=6, r=3, s=3, padding=2, has_bias=True),
 ]
 
 
