@@ -110,12 +110,14 @@ constexpr int CPW = (KC + TS - 1) / TS;      // 32-pixel chunks per wave
 
 // LDS: the two rings while streaming; at the end the same block holds the reduction scratch:
 // per wave NBLK*128 floats for the row-slot halves, the sums of the other waves of a split
-// group, and (atomic publishing) every group's R*S*64 sums in grad_weight order.
+// group, (atomic publishing) every group's R*S*64 sums in grad_weight order, and eight
+// grad_bias sums per wave.
 constexpr int RING_UNITS = NRX * XROW_UNITS + NRD * DROW_UNITS;
 constexpr int SCRATCH_FLOATS = NBLK * 128;  // per wave
 constexpr int RED_FLOATS = GB * (TS - 1) * NBLK * 128;
 constexpr int GROUP_FLOATS = kR * kS * 64;  // grad_weight values of one group
-constexpr int PUBLISH_FLOATS = WAVES * SCRATCH_FLOATS + RED_FLOATS + (SPIO_PARTIALS ? 0 : GB * GROUP_FLOATS);
+constexpr int PUBLISH_FLOATS = WAVES * SCRATCH_FLOATS + RED_FLOATS + (SPIO_PARTIALS ? 0 : GB * GROUP_FLOATS) +
+                               (SPIO_HAS_BIAS ? WAVES * 8 : 0);
 constexpr int LDS_UNITS = RING_UNITS > (PUBLISH_FLOATS + 3) / 4 ? RING_UNITS : (PUBLISH_FLOATS + 3) / 4;
 static_assert(LDS_UNITS * 16 <= 160 * 1024, "LDS overflow");
 static_assert(NRD % 2 == 0 && NRD >= kR + 1, "dy ring too small");
@@ -496,26 +498,6 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
 #endif
             if (TS > 1) block_sync();  // the scratch is rewritten for the next filter row
         }
-#if SPIO_HAS_BIAS
-        // grad_bias[8g + k] = accb of row slot 0 (lanes 0-31) + row slot 1 (lanes 32-63); every
-        // column holds the same sum, lanes 0 and 16 publish channels 0-3 and 4-7.
-        {
-            if (lane >= 32) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) scratch[e * 32 + (lane - 32)] = accb[e];
-            }
-            float tb[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                tb[e] = 0.f;
-                if (lane < 32) tb[e] = accb[e] + scratch[e * 32 + lane];
-            }
-            if (wave_active && grad_bias != nullptr && (lane & 47) == 0) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) atomic_add_f32(grad_bias + 8 * gglob + k4 + e, tb[e]);
-            }
-        }
-#endif
 #if !SPIO_PARTIALS
         // One wave per group adds the group's R*S*64 sums into grad_weight: every atomic
         // instruction covers 64 consecutive floats (two full 128-byte lines), which the memory
@@ -525,6 +507,35 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
             float* gout = out + (long long)gglob * GROUP_FLOATS;
 #pragma unroll
             for (int i = 0; i < kR * kS; ++i) atomic_add_f32(gout + 64 * i + lane, gstage[64 * i + lane]);
+        }
+#endif
+#if SPIO_HAS_BIAS
+        // grad_bias[8g + k] = accb of row slot 0 (lanes 0-31) + row slot 1 (lanes 32-63); every
+        // column holds the same sum, so lanes 0 and 16 carry channels 0-3 and 4-7.  All waves
+        // leave their eight sums in LDS and one wave adds the workgroup's GB*8 consecutive
+        // values with a single atomic instruction: atomics of different workgroups to the same
+        // 128-byte line retire one after the other, so their number per line is what counts.
+        {
+            if (lane >= 32) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) scratch[e * 32 + (lane - 32)] = accb[e];
+            }
+            float* bslots = reinterpret_cast<float*>(lds) + WAVES * SCRATCH_FLOATS + RED_FLOATS +
+                            (SPIO_PARTIALS ? 0 : GB * GROUP_FLOATS);  // [wave][8]
+            if ((lane & 47) == 0) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    bslots[wave * 8 + k4 + e] = wave_active ? accb[e] + scratch[e * 32 + lane] : 0.f;
+            }
+            block_sync();
+            if (wave == 0 && grad_bias != nullptr) {
+                for (int i = lane; i < GB * 8; i += 64) {
+                    float v = 0.f;
+#pragma unroll
+                    for (int w2 = 0; w2 < TS; ++w2) v += bslots[(w2 * GB + i / 8) * 8 + (i & 7)];
+                    if (cb * GB + i / 8 < kGroups) atomic_add_f32(grad_bias + 8 * cb * GB + i, v);
+                }
+            }
         }
 #endif
     }

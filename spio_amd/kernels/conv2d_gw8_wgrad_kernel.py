@@ -30,7 +30,7 @@ MAX_WAVES = 16
 MAX_LDS_BYTES = 128 * 1024
 MAX_LOADS_PER_THREAD = 8
 MAX_ACCUMULATORS = 32
-MAX_GEOMETRIES = 12
+MAX_GEOMETRIES = 16
 PIPELINE_CHOICES = ((2, 1), (4, 1), (2, 2))  # (prefetch, rows)
 
 
@@ -88,7 +88,8 @@ def wgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig) -> Dic
     # the same LDS block holds the reduction scratch at the end: per-wave row-slot halves, the
     # sums of the other waves of a split group, and (atomic publishing) every group's R*S*64 sums
     lds_scratch = (gb * ts * (s2 // 2) * 128 + gb * (ts - 1) * (s2 // 2) * 128
-                   + (0 if config.two_stage else gb * r * s * 64)) * 4  # fmt: skip
+                   + (0 if config.two_stage else gb * r * s * 64)
+                   + (gb * ts * 8 if params.has_bias else 0)) * 4  # fmt: skip
     g = dict(
         NBLK=s2 // 2, ND=r + 1, WPI=wpi, F=f, KC=kc, GSX=gsx, GSD=gsd, NRD=nrd, THREADS=threads,
         LDS_BYTES=max(lds_rings, lds_scratch), RING_BYTES=lds_rings, SCRATCH_BYTES=lds_scratch,
