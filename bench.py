@@ -39,9 +39,9 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what
 # the same counter reads for the plain copy kernel (profiles/conv2d_gw8_target_hbm_traffic.md).
 MEASURED_TRAFFIC_BYTES = {
-    ("target", "fprop"): 103_670_000,
-    ("target", "dgrad"): 103_650_000,
-    ("target", "wgrad"): 105_890_000,
+    ("target", "fprop"): 104_710_000,
+    ("target", "dgrad"): 104_720_000,
+    ("target", "wgrad"): 105_510_000,
 }
 CACHE_BYTES = 256 * 1024 * 1024
 
