@@ -9,9 +9,9 @@
 // Design
 //   * A workgroup owns SPIO_BH rows of dy (output rows) of SPIO_NB images side
 //     by side, for SPIO_GB channel groups, and repeats that for SPIO_ITERS
-//     image blocks before it publishes its sums.  Per step it stages one row
-//     of x and one row of dy in LDS ([group][flattened pixel][8 ch], zero
-//     halo materialised once, as in the forward kernel).
+//     image blocks before it publishes its sums.  Per step it stages SPIO_RB
+//     (1 or 2) rows of x and of dy in LDS ([group][flattened pixel][8 ch],
+//     zero halo materialised once, as in the forward kernel).
 //   * One wave owns one group.  The contraction runs over pixels, so both MFMA
 //     operands need "8 pixels of one channel" per lane while memory holds
 //     "8 channels of one pixel"; the transposing LDS read of gfx950
@@ -19,22 +19,28 @@
 //   * v_mfma_f32_16x16x32_f16 per 32-pixel chunk:
 //         A (16 x 32) = dy:  rows m = 8*j + k    (two dy rows j of an aligned row pair, 8 k)
 //         B (32 x 16) = x:   cols n = 8*sj + c   (two column taps sj, 8 c)
-//     so one MFMA yields dw for 2 filter rows x 2 filter columns.  For the x
-//     row of step t and the dy row pair (2i, 2i+1) the filter rows are
-//     r = delta - j with delta = t - 2i in [0, R]; there is one accumulator per
-//     (delta, column-tap pair).  Entries with r or s out of range are never read.
+//     so one MFMA yields dw for 2 filter rows x 2 filter columns.  For x row t
+//     and the dy row pair (2i, 2i+1) the filter rows are r = delta - j with
+//     delta = t - 2i in [0, R]; there is one accumulator per (delta, column-tap
+//     pair).  Entries with r or s out of range are never read.
 //   * At the end dw[k,r,s,c] = acc[delta=r] (lanes with j=0) + acc[delta=r+1]
-//     (lanes with j=1); the halves are combined through LDS.  fp32 atomics are
-//     the scarce resource (the device retires roughly 128 per clock in total,
-//     and every workgroup owes R*S*64 of them per group), so there are two
-//     ways to publish: SPIO_PARTIALS=0 adds straight into grad_weight with
-//     atomics; SPIO_PARTIALS=1 stores each workgroup's sums into its own
-//     partial image of a workspace with plain stores, and the small
-//     <name>_reduce kernel below folds the partial images into grad_weight.
-//     (Reducing inside the kernel by "the last workgroup of a group to finish"
-//     was measured and rejected: the device-scope release/acquire fences it
-//     needs write back and invalidate the L2 of an XCD and cost more than the
-//     atomics they save.)
+//     (lanes with j=1); the halves are combined through LDS.  Two ways to
+//     publish: SPIO_PARTIALS=0 adds into grad_weight with fp32 atomics.  Atomics
+//     of different workgroups to the same 128-byte line retire one after the
+//     other, so the sums are first staged in LDS in grad_weight order and then
+//     added with instructions that cover 64 consecutive floats (two full
+//     lines): the fewest line operations possible.  SPIO_PARTIALS=1 stores each
+//     workgroup's sums into its own partial image of a workspace with plain
+//     stores, and the small <name>_reduce kernel below folds the partial images
+//     into grad_weight.  (Reducing inside the kernel by "the last workgroup of
+//     a group to finish" was measured and rejected: the device-scope
+//     release/acquire fences it needs write back and invalidate the L2 of an
+//     XCD and cost more than the atomics they save.)
+//   * With SPIO_HAS_BIAS the kernel takes a fourth pointer, grad_bias ([K]
+//     fp32, accumulated into like grad_weight; null = not wanted), and sums dy
+//     per channel in the same pass: one more MFMA per chunk and row pair with
+//     an all-ones B operand (the reference runs a separate reduction,
+//     spio/functional/conv2d_gw8_function.py:134-136).
 #include "spio_conv_common.h"
 
 using namespace spio;
