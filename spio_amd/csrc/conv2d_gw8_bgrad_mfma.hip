@@ -1,0 +1,595 @@
+// Fused backward kernel for conv2d_gw8 (gfx950): data gradient and weight gradient (and,
+// optionally, the bias gradient) in one pass.
+//
+// Contract (reference kernels: spio/src/conv2d_gw8.cu:10-225 in its data-gradient mode and
+// spio/src/conv2d_gw8_wgrad.cu:10-226; the reference launches them one after the other,
+// spio/functional/conv2d_gw8_function.py:119-146):
+//   dx[n,h,w,8g+c] = rn16(sum_{j,r,s} dy[n,h-r+py,w-s+px,8g+j] * w[8g+j,r,s,c])
+//   dw[k,r,s,c]   += sum_{n,p,q} x[n,p+r-py,q+s-px,8g+c] * dy[n,p,q,k]            (fp32, atomics)
+//   db[k]         += sum_{n,p,q} dy[n,p,q,k]                                      (with a bias)
+//
+// Why fuse: both gradients stream grad_output.  Run separately they move
+// 2*|dy| + |x| + |dx| bytes through HBM; fused, dy is read once: 25 % less traffic for the
+// backward step of an HBM-bound operator, and one launch instead of two.
+//
+// Scope: "same" convolutions only (2*py = R-1, 2*px = S-1, so P = H and Q = W): then one copy
+// of a dy row in LDS serves both gradients, and the dx row that completes at a step has the
+// index of the x row of that step.  A workgroup owns whole images (all rows) of SPIO_NB images
+// side by side for SPIO_GB channel groups, repeated for SPIO_ITERS image blocks, so no dx row
+// needs dy rows of another workgroup.  Everything else is the separate kernels' design:
+//   * rows of x and dy staged in LDS as [group][flattened pixel][8 ch], zero halo materialised
+//     once, branch-free global loads SPIO_PF steps ahead;
+//   * weight gradient: A = dy row pair, B = x (two column taps), one accumulator per (delta,
+//     tap pair), transposing LDS reads (see conv2d_gw8_wgrad_mfma.hip);
+//   * data gradient: A = flipped, group-transposed filter, B = dy (pixel n + tap kb is the
+//     16 bytes lane (n, kb) reads), rotating accumulator row slots (see conv2d_gw8_mfma.hip);
+//     a dy pixel (image i, column q) sits at flattened pixel i*WPI + q + px, which is both its
+//     place as a source pixel of the data gradient and, shifted by px, its place opposite x in
+//     the weight gradient;
+//   * publishing of dw (and db) as in the weight-gradient kernel: sums staged in LDS in
+//     grad_weight order, atomics of 64 consecutive floats.
+#include "spio_conv_common.h"
+
+using namespace spio;
+
+#ifndef SPIO_NB
+#define SPIO_NB 1
+#endif
+#ifndef SPIO_ITERS
+#define SPIO_ITERS 1
+#endif
+#ifndef SPIO_PF
+#define SPIO_PF 2
+#endif
+#ifndef SPIO_TS
+#define SPIO_TS 1
+#endif
+#ifndef SPIO_HAS_BIAS
+#define SPIO_HAS_BIAS 0
+#endif
+
+namespace {
+
+static_assert(2 * kPadY == kR - 1 && 2 * kPadX == kS - 1, "the fused backward kernel needs P = H and Q = W");
+
+constexpr int GB = SPIO_GB;        // groups per workgroup
+constexpr int NB = SPIO_NB;        // images side by side
+constexpr int ITERS = SPIO_ITERS;  // image blocks per workgroup
+constexpr int TS = SPIO_TS;        // waves per group: they split the 32-pixel chunks and the 16-pixel tiles
+constexpr int PF = SPIO_PF;        // prefetch distance in rows (even)
+constexpr int WAVES = GB * TS;
+constexpr int THREADS = 64 * WAVES;
+constexpr bool kDbias = SPIO_HAS_BIAS != 0;
+
+// ---- weight gradient ----
+constexpr int S2 = 2 * ((kS + 1) / 2);
+constexpr int NBLK = S2 / 2;          // column-tap pairs
+constexpr int ND = kR + 1;            // values of delta
+constexpr int NPAIR = kR / 2 + 1;     // aligned dy row pairs one x row meets
+constexpr int WPI = kW + kS - 1;      // padded width of one image
+constexpr int F = NB * WPI;           // flattened pixels of a staged row
+constexpr int KSPAN = (NB - 1) * WPI + kQ;
+constexpr int KC = (KSPAN + 31) / 32;     // 32-pixel chunks
+constexpr int CPW = (KC + TS - 1) / TS;   // chunks per wave
+// ---- data gradient ----
+constexpr int NS = 2 * ((kR + 1) / 2);   // accumulator row slots
+constexpr int NACC = NS / 2;
+constexpr int KB = (kS + 3) / 4;         // MFMA K-steps per dy row (4 column taps each)
+constexpr int WT = (F - kS + 1 + 15) / 16;   // 16-pixel tiles of a dx row
+constexpr int TPW = (WT + TS - 1) / TS;      // tiles per wave
+// ---- LDS geometry ----
+constexpr int FPX = 32 * KC + S2 - 1;  // x pixels a weight-gradient read can touch
+constexpr int GSX = FPX + ((9 - FPX % 16) + 16) % 16;  // x group stride (pixels), = 9 mod 16
+constexpr int FPD_W = kPadX + 32 * KC;                 // dy pixels: weight-gradient reads
+constexpr int FPD_D = 16 * WT + 4 * KB - 1;            // dy pixels: data-gradient reads
+constexpr int FPD = FPD_W > FPD_D ? FPD_W : FPD_D;
+constexpr int GSD = FPD + ((9 - FPD % 16) + 16) % 16;  // dy group stride, = 9 mod 16
+constexpr int NRX = 2;                                 // x ring rows
+constexpr int NRD = 2 * ((kR + 2) / 2);                // dy ring rows: even, >= R+1
+constexpr int XROW_UNITS = GB * GSX;
+constexpr int DROW_UNITS = GB * GSD + ((4 - (GB * GSD) % 16) + 16) % 16;
+constexpr int OSTRIDE = GB * 16 + 16;        // bytes per pixel in the dx output stage
+constexpr int OUT_ROW_BYTES = 16 * WT * OSTRIDE;
+constexpr int X_CELLS = F * GB;
+constexpr int LPTX = (X_CELLS + THREADS - 1) / THREADS;
+constexpr int D_CELLS = NB * kQ * GB;
+constexpr int LPTD = (D_CELLS + THREADS - 1) / THREADS;  // dy loads = dx stores per thread per row
+constexpr int GBLKS = (kGroups + GB - 1) / GB;
+constexpr int NBLKS = (kN + NB * ITERS - 1) / (NB * ITERS);
+constexpr int NUM_BLOCKS = GBLKS * NBLKS;
+// steps: x rows -py .. H-1+py.  The bias sum takes a dy row pair one step after its first row
+// was staged, so a one-row filter needs one more step when the sum is wanted.
+constexpr int ROWS = kP + (SPIO_HAS_BIAS && kR == 1 ? 2 : kR) - 1;
+
+constexpr int gcd_(int a, int b) { return b == 0 ? a : gcd_(b, a % b); }
+constexpr int UNROLL = NS / gcd_(NS, PF) * PF;  // lcm(NS, PF): even
+constexpr int pmod(int a, int m) { return ((a % m) + m) % m; }
+
+constexpr int RING_UNITS = NRX * XROW_UNITS + NRD * DROW_UNITS;
+constexpr int STREAM_UNITS = RING_UNITS + 2 * OUT_ROW_BYTES / 16;
+constexpr int FILTER_UNITS = GB * 8 * kR * kS;  // filters staged once at the start
+constexpr int SCRATCH_FLOATS = NBLK * 128;      // per wave: row-slot halves
+constexpr int RED_FLOATS = GB * (TS - 1) * NBLK * 128;
+constexpr int GROUP_FLOATS = kR * kS * 64;
+constexpr int PUBLISH_FLOATS =
+    WAVES * SCRATCH_FLOATS + RED_FLOATS + GB * GROUP_FLOATS + (SPIO_HAS_BIAS ? WAVES * 8 : 0);
+constexpr int max3(int a, int b, int c) { return a > b ? (a > c ? a : c) : (b > c ? b : c); }
+constexpr int LDS_UNITS = max3(STREAM_UNITS, FILTER_UNITS, (PUBLISH_FLOATS + 3) / 4);
+static_assert(LDS_UNITS * 16 <= 160 * 1024, "LDS overflow");
+static_assert(PF >= 2 && PF % 2 == 0 && WAVES <= 16, "bad configuration");
+
+SPIO_DEVICE spio_half8 read_tr_pair(const unsigned char* lo, const unsigned char* hi) {
+    typedef spio_short4 __attribute__((address_space(3))) * lds_ptr;
+    union {
+        spio_short4 s[2];
+        spio_half8 h;
+    } v;
+    v.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)lo);
+    v.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)hi);
+    return v.h;
+}
+
+}  // namespace
+
+extern "C" __global__ void SPIO_LAUNCH_BOUNDS(THREADS)
+SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_weight,
+                 const spio_uint4* __restrict__ x, const spio_uint4* __restrict__ dy,
+                 const spio_half* __restrict__ weights
+#if SPIO_HAS_BIAS
+                 , float* __restrict__ grad_bias  // [K] fp32, accumulated into; null = not wanted
+#endif
+) {
+    // One LDS block: x ring, dy ring, two dx output-stage rows.  Before the first row it holds
+    // the staged filters, after the last one the reduction scratch.
+    __shared__ spio_uint4 lds[LDS_UNITS];
+    spio_uint4* const xring = lds;
+    spio_uint4* const dring = lds + NRX * XROW_UNITS;
+    unsigned char* const ostage = reinterpret_cast<unsigned char*>(lds + RING_UNITS);
+
+    const int tid = thread_id();
+    const int lane = tid & 63;
+    // scalar wave index: conditions on it become scalar branches, so no MFMA (which ignores the
+    // lane mask) is issued under an empty mask
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wg = wave % GB;
+    const int ws = wave / GB;
+
+    int b = block_id();
+    if (NUM_BLOCKS % 8 == 0) b = (b & 7) * (NUM_BLOCKS / 8) + (b >> 3);
+    const int cb = b % GBLKS;
+    const int nbk = b / GBLKS;
+    const int gglob = cb * GB + wg;
+    const bool wave_active = gglob < kGroups;
+
+    // ---- data-gradient filter fragments: wfrag[d][u], d = (phase - 2*acc) mod NS ----
+    // A[m = dx channel ch][jj] = w[8g+jj][R-1-r][S-1-s][ch].  The workgroup copies its groups'
+    // filters to LDS as they lie in memory and every wave reads its fragments with the
+    // transposing LDS read (same scheme as the data-gradient mode of conv2d_gw8_mfma.hip).
+    spio_half8 wfrag[NS][KB];
+    {
+        for (int i = tid; i < FILTER_UNITS; i += THREADS) {
+            const int g = i / (8 * kR * kS);
+            const int rem = i % (8 * kR * kS);
+            spio_uint4 v = spio_uint4{0u, 0u, 0u, 0u};
+            if (cb * GB + g < kGroups)
+                v = reinterpret_cast<const spio_uint4*>(weights)[(long long)(cb * GB + g) * (8 * kR * kS) + rem];
+            lds[i] = v;
+        }
+        block_sync();
+        const int kbl = lane >> 4;
+        const int jr = (lane & 15) >> 2;
+        const int t4 = lane & 3;
+        const int src_slot = t4 >> 1;
+        const int my_slot = (lane & 15) >> 3;
+        typedef spio_short4 __attribute__((address_space(3))) * lds_ptr;
+#pragma unroll
+        for (int d = 0; d < NS; ++d) {
+#pragma unroll
+            for (int u = 0; u < KB; ++u) {
+                const int s = 4 * u + kbl;
+                const int r_src = (d - src_slot + NS) % NS;
+                const int r_mine = (d - my_slot + NS) % NS;
+                const int rr = r_src < kR ? kR - 1 - r_src : 0;  // dead taps: any valid address
+                const int ss = s < kS ? kS - 1 - s : 0;
+                const unsigned char* base = reinterpret_cast<const unsigned char*>(lds) +
+                                            ((((wg * 8 + jr) * kR + rr) * kS + ss) * 16) + (t4 & 1) * 8;
+                union {
+                    spio_short4 q[2];
+                    spio_half8 h;
+                } v;
+                v.q[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)base);
+                v.q[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(base + 4 * kR * kS * 16));
+                if (!(wave_active && r_mine < kR && s < kS)) v.h = spio_half8{0, 0, 0, 0, 0, 0, 0, 0};
+                wfrag[d][u] = v.h;
+            }
+        }
+        block_sync();  // everyone has its fragments before the rings are zero-filled
+    }
+
+    // ---- lane roles ----
+    // weight gradient (transposing reads): block kb = lane/16 covers pixels 8*kb..8*kb+7, source
+    // lane 4*jr + t supplies pixel jr (+4 for the second read) of unit t/2 (dy row j or column
+    // tap sj) and channel half t%2.
+    const int kb = lane >> 4;
+    const int jr = (lane & 15) >> 2;
+    const int tt = lane & 3;
+    const int sel = tt >> 1;
+    const int xfrag_off = ((wg * GSX + 8 * kb + jr + sel) * 16) + (tt & 1) * 8;
+    const int dfrag_off = ((wg * GSD + kPadX + 8 * kb + jr) * 16) + (tt & 1) * 8;
+    // data gradient: D[m = 4*(lane/16)+i][n = lane%16]: pixel n, row slot lane/32, channels
+    // 4*((lane/16)&1) + i
+    const int out_j = lane >> 5;
+    const int out_kh = (lane >> 4) & 1;
+    const int out_n = lane & 15;
+
+    spio_float4 acc[ND][NBLK];  // weight gradient
+#pragma unroll
+    for (int d = 0; d < ND; ++d)
+#pragma unroll
+        for (int nb = 0; nb < NBLK; ++nb) acc[d][nb] = spio_float4{0.f, 0.f, 0.f, 0.f};
+    spio_float4 accb = spio_float4{0.f, 0.f, 0.f, 0.f};  // bias gradient
+    const spio_half8 ones8 = spio_half8{1, 1, 1, 1, 1, 1, 1, 1};
+    (void)ones8;
+
+    const long long row_units = (long long)kW * kGroups;  // 16-byte units per row of x, dy and dx
+    const spio_uint4 zero4 = spio_uint4{0u, 0u, 0u, 0u};
+
+    for (int it = 0; it < ITERS; ++it) {
+        const int n0 = (nbk * ITERS + it) * NB;
+        if (n0 >= kN) break;
+
+        // ---- loop-invariant addressing for this image block (branch-free loads: cells without
+        //      data load a valid address and become zero when written to LDS) ----
+        int x_off[LPTX], x_lds[LPTX];
+        bool x_ok[LPTX];
+        const int dummy = n0 * kH * kW * kGroups;
+#pragma unroll
+        for (int l = 0; l < LPTX; ++l) {
+            const int cell = tid + THREADS * l;
+            x_off[l] = dummy;
+            x_ok[l] = false;
+            x_lds[l] = -1;
+            if (cell < X_CELLS) {
+                const int g = cell % GB;
+                const int f = cell / GB;
+                const int img = f / WPI;
+                const int col = f % WPI - kPadX;
+                x_lds[l] = g * GSX + f;
+                if (col >= 0 && col < kW && n0 + img < kN && cb * GB + g < kGroups) {
+                    x_off[l] = ((n0 + img) * kH * kW + col) * kGroups + cb * GB + g;
+                    x_ok[l] = true;
+                }
+            }
+        }
+        // dy cells, and the dx cells of the same (image, column, group): same global offset
+        int d_off[LPTD], d_lds[LPTD], o_lds[LPTD];
+        bool d_ok[LPTD];
+#pragma unroll
+        for (int l = 0; l < LPTD; ++l) {
+            const int cell = tid + THREADS * l;
+            d_off[l] = dummy;
+            d_ok[l] = false;
+            d_lds[l] = -1;
+            o_lds[l] = 0;
+            if (cell < D_CELLS) {
+                const int g = cell % GB;
+                const int q = (cell / GB) % kQ;
+                const int img = cell / (GB * kQ);
+                d_lds[l] = g * GSD + img * WPI + q + kPadX;
+                o_lds[l] = (img * WPI + q) * OSTRIDE + g * 16;
+                if (n0 + img < kN && cb * GB + g < kGroups) {
+                    d_off[l] = ((n0 + img) * kP * kQ + q) * kGroups + cb * GB + g;
+                    d_ok[l] = true;
+                }
+            }
+        }
+
+        // ---- prologue: rows 0..PF-1 into registers ----
+        spio_uint4 xpre[PF][LPTX], dpre[PF][LPTD];
+#pragma unroll
+        for (int t = 0; t < PF; ++t) {
+            const int h = imin(imax(t - kPadY, 0), kH - 1);
+#pragma unroll
+            for (int l = 0; l < LPTX; ++l) xpre[t][l] = load_stream(x + x_off[l] + h * row_units);
+            const int pr = imin(t, kP - 1);
+#pragma unroll
+            for (int l = 0; l < LPTD; ++l) dpre[t][l] = load_stream(dy + d_off[l] + pr * row_units);
+        }
+        if (it == 0) {
+            // zero both rings once, while the first loads are in flight: halo, gap and slack
+            // cells are never written again
+            for (int i = tid; i < RING_UNITS; i += THREADS) lds[i] = zero4;
+        }
+        block_sync();  // rings zeroed / previous image block finished
+        {
+            const bool xrow_ok = -kPadY >= 0;  // x row of step 0 is row -py
+#pragma unroll
+            for (int l = 0; l < LPTX; ++l)
+                if (x_lds[l] >= 0) xring[x_lds[l]] = (xrow_ok && x_ok[l]) ? xpre[0][l] : zero4;
+#pragma unroll
+            for (int l = 0; l < LPTD; ++l)
+                if (d_lds[l] >= 0) dring[d_lds[l]] = d_ok[l] ? dpre[0][l] : zero4;
+        }
+        block_sync();
+
+        spio_float4 dacc[TPW][NACC];  // data gradient: rotating row slots
+#pragma unroll
+        for (int i = 0; i < TPW; ++i)
+#pragma unroll
+            for (int a = 0; a < NACC; ++a) dacc[i][a] = spio_float4{0.f, 0.f, 0.f, 0.f};
+
+        // Coalesced store of the dx row staged at step `ts` (row ts - py), one step later.
+        auto store_dx_row = [&](int ts, int obuf) {
+            const int h = ts - kPadY;
+            if (h >= 0 && h < kH) {
+#pragma unroll
+                for (int l = 0; l < LPTD; ++l) {
+                    if (d_ok[l]) {
+                        const spio_uint4 v =
+                            *reinterpret_cast<const spio_uint4*>(ostage + obuf * OUT_ROW_BYTES + o_lds[l]);
+                        store_stream(v, grad_input + d_off[l] + h * row_units);
+                    }
+                }
+            }
+        };
+
+        for (int tb = 0; tb < ROWS; tb += UNROLL) {
+#pragma unroll
+            for (int uu = 0; uu < UNROLL; ++uu) {
+                const int t = tb + uu;
+                if (t >= ROWS) break;
+                const int sp = uu & 1;                   // parity of t: x ring row, parity of delta
+                const int pbuf = uu % PF;                // register buffer that held row t
+                const int ph = pmod(uu + kPadY, NS);     // data-gradient phase: (t + py) mod NS
+                const int obuf = uu & 1;
+
+                // 1. fragment reads: x row t - py, the dy row pairs it meets, dy row t as the
+                //    data gradient's source row
+                const int hcur = t - kPadY;
+                const bool x_live = hcur >= 0 && hcur < kH;
+                const bool d_live = t < kP;  // dy row t exists
+                const int tbase = t - sp;
+                const bool bias_pair = kDbias && sp == 1 && tbase < kP;
+                const bool do_w = wave_active && (x_live || bias_pair);
+                spio_half8 bfrag[CPW][NBLK], afrag[CPW][NPAIR];
+                if (do_w) {
+#pragma unroll
+                    for (int ci = 0; ci < CPW; ++ci) {
+                        const int ch = ws + TS * ci;
+                        if (TS > 1 && ch >= KC) break;
+                        const unsigned char* xrow =
+                            reinterpret_cast<const unsigned char*>(xring + sp * XROW_UNITS) + xfrag_off;
+#pragma unroll
+                        for (int nb = 0; nb < NBLK; ++nb) {
+                            const unsigned char* pb0 = xrow + (32 * ch + 2 * nb) * 16;
+                            bfrag[ci][nb] = read_tr_pair(pb0, pb0 + 4 * 16);
+                        }
+#pragma unroll
+                        for (int m = 0; m < NPAIR; ++m) {
+                            const int i2 = tbase - 2 * m;
+                            if (i2 >= 0 && i2 < kP) {
+                                const int slot = (i2 + sel) % NRD;
+                                const unsigned char* pa0 =
+                                    reinterpret_cast<const unsigned char*>(dring + slot * DROW_UNITS) +
+                                    dfrag_off + (32 * ch) * 16;
+                                afrag[ci][m] = read_tr_pair(pa0, pa0 + 4 * 16);
+                            }
+                        }
+                    }
+                }
+                const bool do_d = wave_active && d_live;
+                spio_half8 sfrag[TPW][KB];
+                if (do_d) {
+                    const spio_uint4* rrow =
+                        dring + (t % NRD) * DROW_UNITS + wg * GSD + (lane & 15) + (lane >> 4);
+#pragma unroll
+                    for (int i = 0; i < TPW; ++i) {
+                        const int tile = ws + TS * i;
+                        if (TS == 1 || tile < WT) {
+#pragma unroll
+                            for (int u = 0; u < KB; ++u) {
+                                Pack16 v;
+                                v.u = rrow[16 * tile + 4 * u];
+                                sfrag[i][u] = v.h;
+                            }
+                        }
+                    }
+                }
+
+                // 2. prefetch rows t+PF (rows past the end repeat a real row and are never used)
+                {
+                    const int t2 = t + PF;
+                    const int h = imin(imax(t2 - kPadY, 0), kH - 1);
+#pragma unroll
+                    for (int l = 0; l < LPTX; ++l) xpre[pbuf][l] = load_stream(x + x_off[l] + h * row_units);
+                    const int pr = imin(t2, kP - 1);
+#pragma unroll
+                    for (int l = 0; l < LPTD; ++l) dpre[pbuf][l] = load_stream(dy + d_off[l] + pr * row_units);
+                }
+
+                // 3. the dx row finished in the previous step goes out
+                store_dx_row(t - 1, (uu + 1) & 1);
+
+                // 4. rows t+1 into LDS (dy rows past the last one become zero).  The ring rows
+                //    written here are not read in this step, except for dy entries of the weight
+                //    gradient whose filter row is out of range and whose product is ignored.
+                if (t + 1 < ROWS) {
+                    const int hn = t + 1 - kPadY;
+                    if (hn >= 0 && hn < kH) {
+#pragma unroll
+                        for (int l = 0; l < LPTX; ++l)
+                            if (x_lds[l] >= 0)
+                                xring[((sp + 1) & 1) * XROW_UNITS + x_lds[l]] =
+                                    x_ok[l] ? xpre[(uu + 1) % PF][l] : zero4;
+                    }
+                    const int dslot = (t + 1) % NRD;
+                    const bool drow_ok = t + 1 < kP;
+#pragma unroll
+                    for (int l = 0; l < LPTD; ++l)
+                        if (d_lds[l] >= 0)
+                            dring[dslot * DROW_UNITS + d_lds[l]] =
+                                (drow_ok && d_ok[l]) ? dpre[(uu + 1) % PF][l] : zero4;
+                }
+
+                // 5. multiply: weight gradient ...
+                if (do_w) {
+#pragma unroll
+                    for (int ci = 0; ci < CPW; ++ci) {
+                        const int ch = ws + TS * ci;
+                        if (TS > 1 && ch >= KC) break;
+#pragma unroll
+                        for (int m = 0; m < NPAIR; ++m) {
+                            const int i2 = tbase - 2 * m;
+                            if (i2 >= 0 && i2 < kP) {
+                                const int d = sp + 2 * m;  // = t - i2
+                                if (d <= kR && x_live) {
+#pragma unroll
+                                    for (int nb = 0; nb < NBLK; ++nb)
+                                        acc[d][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                            afrag[ci][m], bfrag[ci][nb], acc[d][nb], 0, 0, 0);
+                                }
+                                if (m == 0 && bias_pair)
+                                    accb = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[ci][0], ones8, accb, 0, 0, 0);
+                            }
+                        }
+                    }
+                }
+                //    ... and data gradient: dy row t into the live dx rows
+                if (do_d) {
+#pragma unroll
+                    for (int i = 0; i < TPW; ++i) {
+                        const int tile = ws + TS * i;
+                        if (TS == 1 || tile < WT) {
+#pragma unroll
+                            for (int a = 0; a < NACC; ++a) {
+                                const int d = pmod(ph - 2 * a, NS);
+#pragma unroll
+                                for (int u = 0; u < KB; ++u)
+                                    dacc[i][a] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                        wfrag[d][u], sfrag[i][u], dacc[i][a], 0, 0, 0);
+                            }
+                        }
+                    }
+                }
+
+                // 6. the dx row that received its last tap (row t - py): stage it, reset its slot
+                {
+                    const int slot = pmod(ph - (kR - 1), NS);
+                    const int a = slot >> 1;
+                    const int j = slot & 1;
+                    const bool emit = hcur >= 0 && hcur < kH;
+                    if (wave_active && out_j == j) {
+#pragma unroll
+                        for (int i = 0; i < TPW; ++i) {
+                            const int tile = ws + TS * i;
+                            if (TS == 1 || tile < WT) {
+                                if (emit) {
+                                    Pack8 o;
+#pragma unroll
+                                    for (int e = 0; e < 4; ++e) o.h[e] = (spio_half)dacc[i][a][e];
+                                    *reinterpret_cast<spio_uint2*>(ostage + obuf * OUT_ROW_BYTES +
+                                                                   (16 * tile + out_n) * OSTRIDE + wg * 16 +
+                                                                   out_kh * 8) = o.u;
+                                }
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) dacc[i][a][e] = 0.f;
+                            }
+                        }
+                    }
+                }
+                block_sync();
+            }
+        }
+        store_dx_row(ROWS - 1, (ROWS - 1) & 1);  // the last staged row (if it is a real one)
+    }
+
+    // ---- publish grad_weight (and grad_bias): as in conv2d_gw8_wgrad_mfma.hip ----
+    // dw[k,r,s,c] = acc[delta = r] (lanes 0-31: j = 0) + acc[delta = r+1] (lanes 32-63: j = 1);
+    // the halves meet in a per-wave LDS scratch, the waves of a split group add their sums
+    // through LDS, the group's R*S*64 sums are staged in grad_weight order and added with
+    // atomics of 64 consecutive floats.
+    block_sync();  // every wave is done with the rings and the output stage
+    {
+        float* scratch = reinterpret_cast<float*>(lds) + wave * SCRATCH_FLOATS;
+        float* red = reinterpret_cast<float*>(lds) + WAVES * SCRATCH_FLOATS;
+        float* gstage = reinterpret_cast<float*>(lds) + WAVES * SCRATCH_FLOATS + RED_FLOATS + wg * GROUP_FLOATS;
+        const int k4 = 4 * ((lane >> 4) & 1);
+        const int sj = (lane & 15) >> 3;
+        const int c = lane & 7;
+#pragma unroll
+        for (int r = 0; r < kR; ++r) {
+            float total[NBLK][4];
+#pragma unroll
+            for (int nb = 0; nb < NBLK; ++nb) {
+                if (lane >= 32) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) scratch[e * 32 + (lane - 32)] = acc[r + 1][nb][e];
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    total[nb][e] = 0.f;
+                    if (lane < 32) total[nb][e] = acc[r][nb][e] + scratch[e * 32 + lane];
+                }
+            }
+            if (TS > 1) {
+                if (ws > 0 && lane < 32) {
+#pragma unroll
+                    for (int nb = 0; nb < NBLK; ++nb)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            red[(((wg * (TS - 1) + ws - 1) * NBLK + nb) * 4 + e) * 32 + lane] = total[nb][e];
+                }
+                block_sync();
+                if (ws == 0 && lane < 32) {
+#pragma unroll
+                    for (int w2 = 0; w2 < TS - 1; ++w2)
+#pragma unroll
+                        for (int nb = 0; nb < NBLK; ++nb)
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                total[nb][e] += red[(((wg * (TS - 1) + w2) * NBLK + nb) * 4 + e) * 32 + lane];
+                }
+            }
+            if (wave_active && ws == 0 && lane < 32) {
+#pragma unroll
+                for (int nb = 0; nb < NBLK; ++nb) {
+                    const int s = 2 * nb + sj;
+                    if (s < kS) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) gstage[(((k4 + e) * kR + r) * kS + s) * 8 + c] = total[nb][e];
+                    }
+                }
+            }
+            if (TS > 1) block_sync();  // the scratch is rewritten for the next filter row
+        }
+        if (wave_active && ws == 0) {
+            float* gout = grad_weight + (long long)gglob * GROUP_FLOATS;
+#pragma unroll
+            for (int i = 0; i < kR * kS; ++i) atomic_add_f32(gout + 64 * i + lane, gstage[64 * i + lane]);
+        }
+#if SPIO_HAS_BIAS
+        {
+            if (lane >= 32) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) scratch[e * 32 + (lane - 32)] = accb[e];
+            }
+            float* bslots = reinterpret_cast<float*>(lds) + WAVES * SCRATCH_FLOATS + RED_FLOATS +
+                            GB * GROUP_FLOATS;  // [wave][8]
+            if ((lane & 47) == 0) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    bslots[wave * 8 + k4 + e] = wave_active ? accb[e] + scratch[e * 32 + lane] : 0.f;
+            }
+            block_sync();
+            if (wave == 0 && grad_bias != nullptr) {
+                for (int i = lane; i < GB * 8; i += 64) {
+                    float v = 0.f;
+#pragma unroll
+                    for (int w2 = 0; w2 < TS; ++w2) v += bslots[(w2 * GB + i / 8) * 8 + (i & 7)];
+                    if (cb * GB + i / 8 < kGroups) atomic_add_f32(grad_bias + 8 * cb * GB + i, v);
+                }
+            }
+        }
+#endif
+    }
+}

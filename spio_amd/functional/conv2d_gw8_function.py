@@ -12,18 +12,69 @@ reference (spio/functional/conv2d_gw8_function.py:17-233):
 One deliberate difference: the fake implementation of the backward op reports
 grad_weight as fp32, which is what the real op returns (the reference's fake
 says fp16, :164).
+
+When grad_input and grad_weight are both wanted and the convolution keeps the
+image size, the backward op can run one fused kernel that reads grad_output
+once instead of the reference's two launches (:119-146).  SPIO_FUSED_BACKWARD=0
+never fuses, =1 fuses whenever the shape allows, anything else (default) fuses
+when the recorded kernel times say it is faster, or, without records, when the
+fused kernel has enough workgroups to fill the device.
 """
+
+import os
+import threading
 
 from typing import Tuple
 
 import torch
 
+from ..hip import get_device_attributes
 from ..kernels import (
     Conv2dGw8Params,
+    bgrad_is_supported,
+    conv2d_gw8_bgrad_kernel_factory,
     conv2d_gw8_kernel_factory,
     conv2d_gw8_wgrad_kernel_factory,
+    tuner,
 )
 from ..util import to_channels_last
+
+_fused_choice = {}
+_fused_choice_lock = threading.Lock()
+
+
+def _fused_backward_kernel(params: Conv2dGw8Params, device):
+    """The fused data+weight gradient kernel if it should run for `params`, else None."""
+    mode = os.environ.get("SPIO_FUSED_BACKWARD", "auto").strip().lower()
+    if mode in ("0", "false", "off", "no") or not bgrad_is_supported(params):
+        return None
+    ordinal = device.index if device.index is not None else torch.cuda.current_device()
+    key = (params, ordinal, mode)
+    with _fused_choice_lock:
+        if key in _fused_choice:
+            return _fused_choice[key]
+    attr = get_device_attributes(ordinal)
+    fused = None
+    if list(conv2d_gw8_bgrad_kernel_factory.configs(params, attr)):
+        fused = conv2d_gw8_bgrad_kernel_factory.get_kernel(params, device)
+        if mode not in ("1", "true", "on", "yes"):
+            # the separate kernels, tuned or looked up the same way, for the comparison
+            conv2d_gw8_kernel_factory.get_kernel(params, device, igrad=True)
+            conv2d_gw8_wgrad_kernel_factory.get_kernel(params, device)
+            times = [
+                (tuner.lookup(attr, f.get_full_kernel_name(params, **kw)) or {}).get("us")
+                for f, kw in ((conv2d_gw8_bgrad_kernel_factory, {}),
+                              (conv2d_gw8_kernel_factory, {"igrad": True}),
+                              (conv2d_gw8_wgrad_kernel_factory, {}))
+            ]  # fmt: skip
+            if all(t is not None for t in times):
+                if times[0] >= times[1] + times[2]:
+                    fused = None
+            elif fused.kernel_spec.launch_params.grid[0] < 0.75 * attr.multiprocessor_count:
+                fused = None  # no measurements: too few workgroups to fill the device
+    with _fused_choice_lock:
+        _fused_choice[key] = fused
+    return fused
 
 
 def _is_unit(value) -> bool:
@@ -133,7 +184,19 @@ def conv2d_gw8_backward_op(
     assert tuple(grad_output.shape) == params.output_shape
 
     grad_bias = None
-    if needs_weight_grad:
+    grad_input = None
+    fused = _fused_backward_kernel(params, inputs.device) if needs_input_grad and needs_weight_grad else None
+    if fused is not None:
+        # one pass over grad_output for both gradients (and grad_bias when the layer has a bias)
+        grad_weight = torch.zeros_like(weight, dtype=torch.float32)
+        grad_input = torch.empty_like(inputs)
+        if params.has_bias:
+            if needs_bias_grad:
+                grad_bias = torch.zeros(params.c, dtype=torch.float32, device=inputs.device)
+            fused(grad_input, grad_weight, inputs, grad_output, weight, grad_bias)
+        else:
+            fused(grad_input, grad_weight, inputs, grad_output, weight)
+    elif needs_weight_grad:
         # The kernel accumulates into grad_weight, so it starts from zero; fp32.
         grad_weight = torch.zeros_like(weight, dtype=torch.float32)
         kernel = conv2d_gw8_wgrad_kernel_factory.get_kernel(params, inputs.device)
@@ -151,12 +214,10 @@ def conv2d_gw8_backward_op(
     if needs_bias_grad and grad_bias is None:
         grad_bias = grad_output.sum(dim=(0, 2, 3), dtype=torch.float32)
 
-    if needs_input_grad:
+    if needs_input_grad and grad_input is None:
         grad_input = torch.empty_like(inputs)
         kernel = conv2d_gw8_kernel_factory.get_kernel(params, inputs.device, igrad=True)
         kernel(grad_input, grad_output, weight, None)
-    else:
-        grad_input = None
     return grad_input, grad_weight, grad_bias
 
 

@@ -13,3 +13,8 @@ from .kernel_params_logger import KernelParamsLogger, kernel_params_logging_is_e
 from .tuner import tuner, Tuner
 from .conv2d_gw8_kernel import conv2d_gw8_kernel_factory, Conv2dGw8Config
 from .conv2d_gw8_wgrad_kernel import conv2d_gw8_wgrad_kernel_factory, Conv2dGw8WgradConfig
+from .conv2d_gw8_bgrad_kernel import (
+    conv2d_gw8_bgrad_kernel_factory,
+    Conv2dGw8BgradConfig,
+    bgrad_is_supported,
+)

@@ -1,0 +1,191 @@
+"""Fused backward kernel family of conv2d_gw8: grad_input and grad_weight in one pass.
+
+The reference launches its data-gradient and weight-gradient kernels one after
+the other (spio/functional/conv2d_gw8_function.py:119-146); both stream
+grad_output.  This family reads grad_output once and produces both gradients
+(and grad_bias when the params have a bias), which removes a quarter of the
+backward step's HBM traffic.  It exists for "same" convolutions only
+(2*padding = kernel size - 1 in both directions); `bgrad_is_supported` tells.
+
+Kernel arguments: (grad_input, grad_weight, x, grad_output, weight[, grad_bias]);
+grad_weight (and grad_bias) are accumulated into, so the caller zeroes them first.
+"""
+
+from dataclasses import dataclass, replace
+from typing import Dict, List
+
+import torch
+
+from ..util.math import divup
+from .conv2d_gw8_kernel import _shape_defines
+from .conv2d_gw8_params import Conv2dGw8Params
+from .conv2d_stats import Conv2dStats
+from .kernel import KernelSpec
+from .kernel_factory import KernelFactory
+from .launch_params import LaunchParams
+
+SOURCE = "conv2d_gw8_bgrad_mfma.hip"
+
+MAX_WAVES = 16
+MAX_LDS_BYTES = 128 * 1024
+MAX_LOADS_PER_THREAD = 4
+MAX_REGISTERS = 224  # estimated fragments + accumulators + prefetch buffers, in 32-bit registers
+MAX_GEOMETRIES = 10
+PREFETCH_CHOICES = (2, 4)
+
+
+@dataclass(frozen=True)
+class Conv2dGw8BgradConfig:
+    """Tile configuration of the fused backward kernel.
+
+    Attributes:
+        groups: channel groups per workgroup (one wave each, times `split`).
+        block_n: images whose rows are laid side by side in one staged row.
+        block_n_iters: image blocks a workgroup processes before it publishes grad_weight.
+        prefetch: rows of global loads in flight ahead of the computed row (even).
+        split: waves per group; they share the 32-pixel chunks (weight gradient) and the
+            16-pixel tiles (data gradient) of a row.
+    """
+
+    groups: int = 4
+    block_n: int = 1
+    block_n_iters: int = 1
+    prefetch: int = 4
+    split: int = 1
+
+
+def bgrad_is_supported(params: Conv2dGw8Params) -> bool:
+    """The fused kernel needs output size = input size in both directions."""
+    return 2 * params.padding_h == params.r - 1 and 2 * params.padding_w == params.s - 1
+
+
+def bgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig) -> Dict[str, int]:
+    """Host mirror of the compile-time constants of conv2d_gw8_bgrad_mfma.hip."""
+    r, s = params.r, params.s
+    gb, nb, iters, ts, pf = config.groups, config.block_n, config.block_n_iters, config.split, config.prefetch
+    s2 = 2 * ((s + 1) // 2)
+    nblk = s2 // 2
+    wpi = params.w + s - 1
+    f = nb * wpi
+    kspan = (nb - 1) * wpi + params.q
+    kc = divup(kspan, 32)
+    cpw = divup(kc, ts)
+    ns = 2 * ((r + 1) // 2)
+    kb = divup(s, 4)
+    wt = divup(f - s + 1, 16)
+    tpw = divup(wt, ts)
+    fpx = 32 * kc + s2 - 1
+    gsx = fpx + ((9 - fpx % 16) + 16) % 16
+    fpd = max(params.padding_w + 32 * kc, 16 * wt + 4 * kb - 1)
+    gsd = fpd + ((9 - fpd % 16) + 16) % 16
+    nrd = 2 * ((r + 2) // 2)
+    threads = 64 * gb * ts
+    ring_units = 2 * gb * gsx + nrd * (gb * gsd + ((4 - (gb * gsd) % 16) + 16) % 16)
+    out_row_bytes = 16 * wt * (gb * 16 + 16)
+    stream_bytes = ring_units * 16 + 2 * out_row_bytes
+    filter_bytes = gb * 8 * r * s * 16
+    publish_bytes = (gb * ts * nblk * 128 + gb * (ts - 1) * nblk * 128 + gb * r * s * 64
+                     + (gb * ts * 8 if params.has_bias else 0)) * 4  # fmt: skip
+    lptx = divup(f * gb, threads)
+    lptd = divup(nb * params.q * gb, threads)
+    registers = (
+        4 * ((r + 1) * nblk + 1)  # weight-gradient accumulators (+ bias)
+        + 4 * tpw * (ns // 2)  # data-gradient accumulators
+        + 4 * ns * kb  # filter fragments
+        + 4 * (cpw * (nblk + r // 2 + 1) + tpw * kb)  # operand fragments of one step
+        + 4 * pf * (lptx + lptd)  # prefetch buffers
+    )
+    g = dict(
+        NBLK=nblk, KC=kc, CPW=cpw, WT=wt, TPW=tpw, THREADS=threads,
+        LDS_BYTES=max(stream_bytes, filter_bytes, publish_bytes),
+        LPTX=lptx, LPTD=lptd, REGISTERS=registers,
+        GBLKS=divup(params.groups, gb), NBLKS=divup(params.n, nb * iters),
+        PIXEL_EFF=(nb * params.q) / (32.0 * kc),
+    )  # fmt: skip
+    g["NUM_BLOCKS"] = g["GBLKS"] * g["NBLKS"]
+    return g
+
+
+def _config_is_legal(params, config) -> bool:
+    if not bgrad_is_supported(params):
+        return False
+    g = bgrad_geometry(params, config)
+    return (
+        config.groups * config.split <= MAX_WAVES
+        and config.split <= min(g["KC"], g["WT"])
+        and config.block_n * config.block_n_iters <= max(params.n, 1)
+        and g["LDS_BYTES"] <= MAX_LDS_BYTES
+        and g["LPTX"] <= MAX_LOADS_PER_THREAD
+        and g["REGISTERS"] <= MAX_REGISTERS
+        and config.prefetch >= 2
+        and config.prefetch % 2 == 0
+    )
+
+
+def _score(params, config, num_cus) -> float:
+    """Rough relative cost used only to order (and cap) the sweep; lower is better."""
+    g = bgrad_geometry(params, config)
+    group_eff = params.groups / (g["GBLKS"] * config.groups)
+    quant = divup(g["NUM_BLOCKS"], num_cus) * num_cus / g["NUM_BLOCKS"]
+    stream_us = 6.0 * params.n * params.c * params.h * params.w / 5.0e6
+    publish_us = g["NUM_BLOCKS"] * config.groups * params.r * params.s * 64.0 / (128 * 2.1e3)
+    split_line = 1.0 if (config.groups * 16) % 128 == 0 or config.groups == params.groups else 1.12
+    return (quant * split_line / (g["PIXEL_EFF"] ** 0.3 * group_eff)) * (1.0 + publish_us / stream_us)
+
+
+def _get_configs(params: Conv2dGw8Params, device_attr=None) -> List[Conv2dGw8BgradConfig]:
+    """Legal configurations, most promising first; empty when the shape is not supported."""
+    num_cus = getattr(device_attr, "multiprocessor_count", 256) or 256
+    G = params.groups
+    group_choices = sorted({g for g in (4, 8, 16, G) if g <= min(G, MAX_WAVES)}) or [min(G, MAX_WAVES)]
+    geometries = []
+    for gb in group_choices:
+        for nb in (1, 2, 4, 8):
+            for iters in (1, 2, 4):
+                for ts in (1, 2):
+                    cfg = Conv2dGw8BgradConfig(groups=gb, block_n=nb, block_n_iters=iters, prefetch=2, split=ts)
+                    if _config_is_legal(params, cfg):
+                        geometries.append((_score(params, cfg, num_cus), cfg))
+    geometries.sort(key=lambda sc: sc[0])
+    configs = []
+    for _, base in geometries[:MAX_GEOMETRIES]:
+        for pf in PREFETCH_CHOICES:
+            cfg = replace(base, prefetch=pf)
+            if _config_is_legal(params, cfg):
+                configs.append(cfg)
+    return configs
+
+
+def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig, _device_attr=None) -> KernelSpec:
+    params.validate()
+    assert _config_is_legal(params, config), f"illegal configuration {config} for {params}"
+    g = bgrad_geometry(params, config)
+    defines = _shape_defines(params)
+    defines.update(SPIO_GB=config.groups, SPIO_NB=config.block_n, SPIO_ITERS=config.block_n_iters,
+                   SPIO_PF=config.prefetch, SPIO_TS=config.split,
+                   SPIO_HAS_BIAS=int(params.has_bias))  # fmt: skip
+    return KernelSpec(defines, LaunchParams(grid=g["NUM_BLOCKS"], block=g["THREADS"]), SOURCE, notes=g)
+
+
+def _make_test_args(params: Conv2dGw8Params, device):
+    """Synthetic (grad_input, grad_weight, x, dy, weight[, grad_bias]) for timing."""
+    cl = torch.channels_last
+    x = torch.randn(params.input_shape, device=device, dtype=torch.float16).contiguous(memory_format=cl)
+    dy = torch.randn(params.output_shape, device=device, dtype=torch.float16).contiguous(memory_format=cl)
+    w = torch.randn(params.weight_shape, device=device, dtype=torch.float16).contiguous(memory_format=cl)
+    dx = torch.empty_like(x)
+    dw = torch.zeros(params.weight_shape, device=device, dtype=torch.float32).contiguous(memory_format=cl)
+    if params.has_bias:
+        return (dx, dw, x, dy, w, torch.zeros(params.c, device=device, dtype=torch.float32))
+    return (dx, dw, x, dy, w)
+
+
+conv2d_gw8_bgrad_kernel_factory = KernelFactory(
+    Conv2dGw8Params,
+    Conv2dGw8BgradConfig,
+    Conv2dStats,
+    kernel_name="spio_conv2d_gw8_bgrad",
+    configs=_get_configs,
+    kernel_spec=_get_kernel_spec,
+    make_test_args=_make_test_args,
+)

@@ -33,7 +33,8 @@ def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("shapes", nargs="*", help="shapes in Conv2dGw8Params.encode() form")
     ap.add_argument("--shapes", dest="preset", choices=["bench", "batch-sweep", "network", "all"])
-    ap.add_argument("--directions", default="fprop,dgrad,wgrad")
+    ap.add_argument("--directions", default="fprop,dgrad,wgrad,bgrad",
+                    help="bgrad = the fused data+weight gradient kernel (size-preserving shapes only)")
     ap.add_argument("--iters", type=int, default=30)
     ap.add_argument("--package", action="store_true", help="write into spio_amd/kernels/tuned/")
     args = ap.parse_args(argv)
@@ -41,7 +42,12 @@ def main(argv=None):
     import torch
 
     from .hip import get_device_attributes
-    from .kernels import Conv2dGw8Params, conv2d_gw8_kernel_factory, conv2d_gw8_wgrad_kernel_factory
+    from .kernels import (
+        Conv2dGw8Params,
+        conv2d_gw8_bgrad_kernel_factory,
+        conv2d_gw8_kernel_factory,
+        conv2d_gw8_wgrad_kernel_factory,
+    )
     from .kernels.tuner import _PACKAGE_RECORDS, device_key, tuner
 
     shapes = list(args.shapes)
@@ -64,6 +70,7 @@ def main(argv=None):
         "fprop": (conv2d_gw8_kernel_factory, {}),
         "dgrad": (conv2d_gw8_kernel_factory, {"igrad": True}),
         "wgrad": (conv2d_gw8_wgrad_kernel_factory, {}),
+        "bgrad": (conv2d_gw8_bgrad_kernel_factory, {}),
     }
     seen = set()
     for shape in shapes:
@@ -73,6 +80,9 @@ def main(argv=None):
         params = Conv2dGw8Params.decode(shape)
         for direction in args.directions.split(","):
             factory, kwargs = families[direction]
+            if not list(factory.configs(params, attr, **kwargs)):
+                print(f"{direction:5s} {shape}: not supported", flush=True)
+                continue
             kernel = tuner.sweep(factory, params, 0, attr, warmup=3, iters=args.iters,
                                  record_path=path, **kwargs)  # fmt: skip
             best = min(r["us"] for r in tuner.last_sweep if "us" in r)

@@ -167,3 +167,37 @@ def run_grad_kernel_test(factory, params: Conv2dGw8Params, configs=None, seed=0,
                 torch.cuda.synchronize()
             oracle.check_close(out, dw_e, acc_depth=depth, what=f"wgrad {params.encode()} {kernel.config}")
         kernel.unload()
+
+
+def run_bgrad_kernel_test(factory, params: Conv2dGw8Params, configs=None, seed=0):
+    """Fused backward kernel: grad_input, grad_weight (and grad_bias) of every picked
+    configuration against the oracle; grad_input is pre-filled with a sentinel."""
+    attr = get_device_attributes(0)
+    x, w, bias, dy = gpu_args(params, seed)
+    dx_e, dw_e, db_e = oracle.grads_torch(x, w, bias, dy, params.padding_h, params.padding_w)
+    picked = pick_configs(factory, params, attr, configs)
+    assert picked, f"no fused backward configuration for {params}"
+    kernels = compile_kernel_configs(factory, params, configs=picked, device_attr=attr)
+    xg, wg, dyg = to_gpu(x), to_gpu(w), to_gpu(dy)
+    d_dx = Conv2dStats(params, output_names="grad_input").accumulation_depths[0]
+    d_dw = Conv2dStats(params, output_names="grad_weight").accumulation_depths[0]
+    for kernel in kernels:
+        kernel.load(0)
+        what = f"{params.encode()} {kernel.config}"
+        dx = torch.full(params.input_shape, DEAD_VALUE, device="cuda", dtype=torch.float16).contiguous(
+            memory_format=torch.channels_last
+        )
+        dw = torch.zeros(params.weight_shape, device="cuda", dtype=torch.float32).contiguous(
+            memory_format=torch.channels_last
+        )
+        if params.has_bias:
+            db = torch.zeros(params.c, device="cuda", dtype=torch.float32)
+            kernel(dx, dw, xg, dyg, wg, db)
+            torch.cuda.synchronize()
+            oracle.check_close(db, db_e, acc_depth=params.n * params.p * params.q, what=f"fused grad_bias {what}")
+        else:
+            kernel(dx, dw, xg, dyg, wg)
+            torch.cuda.synchronize()
+        oracle.check_close(dx, dx_e, acc_depth=d_dx, what=f"fused dgrad {what}")
+        oracle.check_close(dw, dw_e, acc_depth=d_dw, what=f"fused wgrad {what}")
+        kernel.unload()

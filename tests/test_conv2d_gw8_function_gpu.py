@@ -113,6 +113,40 @@ def test_backward_op_skips_what_is_not_needed():
     oracle.check_close(gx, oracle.grads_torch(x, w, b, dy, 1, 1)[0], acc_depth=72, what="dx only")
 
 
+@pytest.mark.parametrize("mode", ["0", "1"])
+def test_backward_op_fused_and_separate_kernels_agree_with_the_oracle(monkeypatch, mode):
+    """SPIO_FUSED_BACKWARD=1 routes the backward op through the fused data+weight(+bias)
+    gradient kernel, =0 through the separate kernels; both must match the oracle."""
+    monkeypatch.setenv("SPIO_FUSED_BACKWARD", mode)
+    for p in (Conv2dGw8Params(n=3, c=40, h=12, w=20, padding=1, has_bias=True),
+              Conv2dGw8Params(n=2, c=16, h=9, w=9, r=5, s=5, padding=2, has_bias=False)):  # fmt: skip
+        x, w, b, dy = oracle.make_args(p.n, p.c, p.h, p.w, p.r, p.s, p.padding_h, p.padding_w, p.has_bias, 3)
+        dx_e, dw_e, db_e = oracle.grads_torch(x, w, b, dy, p.padding_h, p.padding_w)
+        dx, dw, db = torch.ops.spio.conv2d_gw8_backward(
+            to_gpu(x), to_gpu(w), to_gpu(b), to_gpu(dy), p.padding_h, p.padding_w, True, True, p.has_bias
+        )
+        depth = p.n * p.p * p.q
+        oracle.check_close(dx, dx_e, acc_depth=8 * p.r * p.s, what=f"dx mode {mode}")
+        oracle.check_close(dw, dw_e, acc_depth=depth, what=f"dw mode {mode}")
+        if p.has_bias:
+            oracle.check_close(db, db_e, acc_depth=depth, what=f"db mode {mode}")
+
+
+def test_fused_backward_choice(monkeypatch):
+    from spio_amd.functional.conv2d_gw8_function import _fused_backward_kernel
+
+    dev = torch.device("cuda", 0)
+    same = Conv2dGw8Params(n=2, c=16, h=8, w=8, padding=1)
+    monkeypatch.setenv("SPIO_FUSED_BACKWARD", "0")
+    assert _fused_backward_kernel(same, dev) is None
+    monkeypatch.setenv("SPIO_FUSED_BACKWARD", "1")
+    assert _fused_backward_kernel(same, dev) is not None
+    assert _fused_backward_kernel(Conv2dGw8Params(n=2, c=16, h=8, w=8, padding=0), dev) is None
+    # no recorded times for this shape and far fewer workgroups than compute units: separate kernels
+    monkeypatch.setenv("SPIO_FUSED_BACKWARD", "auto")
+    assert _fused_backward_kernel(same, dev) is None
+
+
 def test_wgrad_accumulates_into_its_output():
     """The weight-gradient kernel adds to grad_weight: two launches give exactly twice one
     launch's contribution (up to the order of fp32 atomics)."""

@@ -8,10 +8,13 @@ sentinel.
 
 import pytest
 
-from helpers import run_grad_kernel_test, run_kernel_test, sample_params
+from helpers import run_bgrad_kernel_test, run_grad_kernel_test, run_kernel_test, sample_params
 from spio_amd.kernels import (
+    Conv2dGw8BgradConfig,
     Conv2dGw8Config,
     Conv2dGw8Params,
+    bgrad_is_supported,
+    conv2d_gw8_bgrad_kernel_factory,
     conv2d_gw8_kernel_factory,
     conv2d_gw8_wgrad_kernel_factory,
 )
@@ -49,6 +52,38 @@ def test_dgrad_sanity(params):
 @pytest.mark.parametrize("params", SANITY, ids=lambda p: p.encode())
 def test_wgrad_sanity(params):
     run_grad_kernel_test(conv2d_gw8_wgrad_kernel_factory, params)
+
+
+# size-preserving shapes the fused backward kernel has a configuration for (7x7 needs more
+# registers than a wave has and stays with the separate kernels)
+SAME_SIZE = [p for p in SANITY if bgrad_is_supported(p) and list(conv2d_gw8_bgrad_kernel_factory.configs(p))] + [
+    Conv2dGw8Params(n=5, c=24, h=7, w=9, r=1, s=1, padding=0, has_bias=True),
+    Conv2dGw8Params(n=3, c=16, h=10, w=12, r=5, s=3, padding=(2, 1), has_bias=False),
+    Conv2dGw8Params(n=3, c=72, h=19, w=40, padding=1, has_bias=True),
+]
+
+
+@pytest.mark.parametrize("params", SAME_SIZE, ids=lambda p: p.encode())
+def test_bgrad_sanity(params):
+    """Fused data + weight (+ bias) gradient kernel on the size-preserving shapes."""
+    run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params)
+
+
+def test_bgrad_explicit_configs():
+    """Split groups, images side by side, several image blocks per workgroup, a group count
+    that does not divide the channel blocks, a batch that does not fill the last block."""
+    params = Conv2dGw8Params(n=5, c=48, h=20, w=28, padding=1, has_bias=True)
+    run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params,
+                          configs=[Conv2dGw8BgradConfig(groups=4, block_n=2, block_n_iters=1, prefetch=2, split=2),
+                                   Conv2dGw8BgradConfig(groups=4, block_n=2, block_n_iters=2, prefetch=4, split=1),
+                                   Conv2dGw8BgradConfig(groups=6, block_n=2, block_n_iters=1, prefetch=2, split=2),
+                                   Conv2dGw8BgradConfig(groups=4, block_n=4, block_n_iters=1, prefetch=2, split=2)])  # fmt: skip
+
+
+def test_bgrad_is_not_offered_when_the_image_size_changes():
+    assert not bgrad_is_supported(Conv2dGw8Params(n=1, c=8, h=8, w=8, padding=0))
+    assert not bgrad_is_supported(Conv2dGw8Params(n=1, c=8, h=8, w=8, r=4, s=1, padding=(2, 0)))
+    assert list(conv2d_gw8_bgrad_kernel_factory.configs(Conv2dGw8Params(n=1, c=8, h=8, w=8, padding=2))) == []
 
 
 def test_fprop_explicit_configs():
