@@ -14,9 +14,14 @@
 //
 // Scope: "same" convolutions only (2*py = R-1, 2*px = S-1, so P = H and Q = W): then one copy
 // of a dy row in LDS serves both gradients, and the dx row that completes at a step has the
-// index of the x row of that step.  A workgroup owns whole images (all rows) of SPIO_NB images
-// side by side for SPIO_GB channel groups, repeated for SPIO_ITERS image blocks, so no dx row
-// needs dy rows of another workgroup.  Everything else is the separate kernels' design:
+// index of the x row of that step.  A workgroup owns SPIO_BH rows (of dx, and of dy for the
+// weight gradient) of SPIO_NB images side by side for SPIO_GB channel groups, repeated for
+// SPIO_ITERS image blocks.  It streams the rows p0-py .. p0+BH-1+py of dy and of x: step t
+// stages dy row p0-py+t and x row p0-2py+t (an x row can only be multiplied once the dy rows
+// up to py below it are there).  The py halo rows of dy above and below the block feed the
+// data gradient only; the weight gradient masks them out of its dy fragments, so every dy row
+// is counted by exactly one workgroup.  With SPIO_BH = P a workgroup owns whole images and
+// there is no halo.  Everything else is the separate kernels' design:
 //   * rows of x and dy staged in LDS as [group][flattened pixel][8 ch], zero halo materialised
 //     once, branch-free global loads SPIO_PF steps ahead;
 //   * weight gradient: A = dy row pair, B = x (two column taps), one accumulator per (delta,
@@ -53,6 +58,7 @@ namespace {
 static_assert(2 * kPadY == kR - 1 && 2 * kPadX == kS - 1, "the fused backward kernel needs P = H and Q = W");
 
 constexpr int GB = SPIO_GB;        // groups per workgroup
+constexpr int BH = SPIO_BH;        // rows per workgroup
 constexpr int NB = SPIO_NB;        // images side by side
 constexpr int ITERS = SPIO_ITERS;  // image blocks per workgroup
 constexpr int TS = SPIO_TS;        // waves per group: they split the 32-pixel chunks and the 16-pixel tiles
@@ -96,10 +102,12 @@ constexpr int D_CELLS = NB * kQ * GB;
 constexpr int LPTD = (D_CELLS + THREADS - 1) / THREADS;  // dy loads = dx stores per thread per row
 constexpr int GBLKS = (kGroups + GB - 1) / GB;
 constexpr int NBLKS = (kN + NB * ITERS - 1) / (NB * ITERS);
-constexpr int NUM_BLOCKS = GBLKS * NBLKS;
-// steps: x rows -py .. H-1+py.  The bias sum takes a dy row pair one step after its first row
-// was staged, so a one-row filter needs one more step when the sum is wanted.
-constexpr int ROWS = kP + (SPIO_HAS_BIAS && kR == 1 ? 2 : kR) - 1;
+constexpr int PBLKS = (kP + BH - 1) / BH;
+constexpr int NUM_BLOCKS = GBLKS * PBLKS * NBLKS;
+// steps: dy rows p0-py .. p0+BH-1+py, then py more for the last x rows.  The bias sum takes a dy
+// row pair one step after its first row was staged, so a one-row filter needs one more step
+// when the sum is wanted.
+constexpr int ROWS = BH + 3 * kPadY + (SPIO_HAS_BIAS && kR == 1 ? 1 : 0);
 
 constexpr int gcd_(int a, int b) { return b == 0 ? a : gcd_(b, a % b); }
 constexpr int UNROLL = NS / gcd_(NS, PF) * PF;  // lcm(NS, PF): even
@@ -156,8 +164,14 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
 
     int b = block_id();
     if (NUM_BLOCKS % 8 == 0) b = (b & 7) * (NUM_BLOCKS / 8) + (b >> 3);
-    const int cb = b % GBLKS;
-    const int nbk = b / GBLKS;
+    const int pb = b % PBLKS;
+    const int cb = (b / PBLKS) % GBLKS;
+    const int nbk = b / (PBLKS * GBLKS);
+    const int p0 = pb * BH;
+    const int bh_eff = imin(BH, kP - p0);  // rows this block owns
+    // first and last row (of x and of dy alike) the block needs; loads outside repeat them
+    const int row_lo = imax(p0 - kPadY, 0);
+    const int row_hi = imin(p0 + bh_eff - 1 + kPadY, kP - 1);
     const int gglob = cb * GB + wg;
     const bool wave_active = gglob < kGroups;
 
@@ -288,10 +302,10 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
         spio_uint4 xpre[PF][LPTX], dpre[PF][LPTD];
 #pragma unroll
         for (int t = 0; t < PF; ++t) {
-            const int h = imin(imax(t - kPadY, 0), kH - 1);
+            const int h = imin(imax(p0 - 2 * kPadY + t, row_lo), row_hi);
 #pragma unroll
             for (int l = 0; l < LPTX; ++l) xpre[t][l] = load_stream(x + x_off[l] + h * row_units);
-            const int pr = imin(t, kP - 1);
+            const int pr = imin(imax(p0 - kPadY + t, row_lo), row_hi);
 #pragma unroll
             for (int l = 0; l < LPTD; ++l) dpre[t][l] = load_stream(dy + d_off[l] + pr * row_units);
         }
@@ -302,13 +316,14 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
         }
         block_sync();  // rings zeroed / previous image block finished
         {
-            const bool xrow_ok = -kPadY >= 0;  // x row of step 0 is row -py
+            const bool xrow_ok = kPadY == 0;    // step 0: x row p0 - 2py, needed only without padding
+            const bool drow_ok = p0 - kPadY >= 0;  // step 0: dy row p0 - py
 #pragma unroll
             for (int l = 0; l < LPTX; ++l)
                 if (x_lds[l] >= 0) xring[x_lds[l]] = (xrow_ok && x_ok[l]) ? xpre[0][l] : zero4;
 #pragma unroll
             for (int l = 0; l < LPTD; ++l)
-                if (d_lds[l] >= 0) dring[d_lds[l]] = d_ok[l] ? dpre[0][l] : zero4;
+                if (d_lds[l] >= 0) dring[d_lds[l]] = (drow_ok && d_ok[l]) ? dpre[0][l] : zero4;
         }
         block_sync();
 
@@ -318,10 +333,10 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
 #pragma unroll
             for (int a = 0; a < NACC; ++a) dacc[i][a] = spio_float4{0.f, 0.f, 0.f, 0.f};
 
-        // Coalesced store of the dx row staged at step `ts` (row ts - py), one step later.
+        // Coalesced store of the dx row staged at step `ts` (row p0 - 2py + ts), one step later.
         auto store_dx_row = [&](int ts, int obuf) {
-            const int h = ts - kPadY;
-            if (h >= 0 && h < kH) {
+            const int h = p0 - 2 * kPadY + ts;
+            if (ts >= 2 * kPadY && ts < 2 * kPadY + bh_eff) {
 #pragma unroll
                 for (int l = 0; l < LPTD; ++l) {
                     if (d_ok[l]) {
@@ -340,16 +355,19 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                 if (t >= ROWS) break;
                 const int sp = uu & 1;                   // parity of t: x ring row, parity of delta
                 const int pbuf = uu % PF;                // register buffer that held row t
-                const int ph = pmod(uu + kPadY, NS);     // data-gradient phase: (t + py) mod NS
+                const int ph = uu % NS;                  // data-gradient phase: t mod NS
                 const int obuf = uu & 1;
 
-                // 1. fragment reads: x row t - py, the dy row pairs it meets, dy row t as the
-                //    data gradient's source row
-                const int hcur = t - kPadY;
-                const bool x_live = hcur >= 0 && hcur < kH;
-                const bool d_live = t < kP;  // dy row t exists
+                // 1. fragment reads: x row p0-2py+t, the dy row pairs it meets (dy rows are named
+                //    by the step that staged them: row p0-py+tau at step tau; the block owns
+                //    tau in [py, py+bh_eff)), and dy row p0-py+t as the data gradient's source row
+                const int hcur = p0 - 2 * kPadY + t;
+                const bool x_live = t >= kPadY && hcur >= 0 && hcur < kH;
+                const int dcur = p0 - kPadY + t;
+                const bool d_live = t < bh_eff + 2 * kPadY && dcur >= 0 && dcur < kP;
                 const int tbase = t - sp;
-                const bool bias_pair = kDbias && sp == 1 && tbase < kP;
+                const int own_lo = kPadY, own_hi = kPadY + bh_eff;  // owned dy rows: [own_lo, own_hi)
+                const bool bias_pair = kDbias && sp == 1 && tbase + 1 >= own_lo && tbase < own_hi;
                 const bool do_w = wave_active && (x_live || bias_pair);
                 spio_half8 bfrag[CPW][NBLK], afrag[CPW][NPAIR];
                 if (do_w) {
@@ -366,13 +384,18 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                         }
 #pragma unroll
                         for (int m = 0; m < NPAIR; ++m) {
-                            const int i2 = tbase - 2 * m;
-                            if (i2 >= 0 && i2 < kP) {
-                                const int slot = (i2 + sel) % NRD;
+                            const int i2 = tbase - 2 * m;  // first row of the pair (step numbering)
+                            if (i2 + 1 >= own_lo && i2 < own_hi) {
+                                const int slot = (i2 + sel + NRD) % NRD;
                                 const unsigned char* pa0 =
                                     reinterpret_cast<const unsigned char*>(dring + slot * DROW_UNITS) +
                                     dfrag_off + (32 * ch) * 16;
-                                afrag[ci][m] = read_tr_pair(pa0, pa0 + 4 * 16);
+                                spio_half8 a = read_tr_pair(pa0, pa0 + 4 * 16);
+                                // a halo row in the pair belongs to the neighbouring block; the
+                                // transposed fragment holds row j = (lane % 16) / 8 of the pair
+                                const int row = i2 + ((lane & 15) >> 3);
+                                if (row < own_lo || row >= own_hi) a = spio_half8{0, 0, 0, 0, 0, 0, 0, 0};
+                                afrag[ci][m] = a;
                             }
                         }
                     }
@@ -399,10 +422,10 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                 // 2. prefetch rows t+PF (rows past the end repeat a real row and are never used)
                 {
                     const int t2 = t + PF;
-                    const int h = imin(imax(t2 - kPadY, 0), kH - 1);
+                    const int h = imin(imax(p0 - 2 * kPadY + t2, row_lo), row_hi);
 #pragma unroll
                     for (int l = 0; l < LPTX; ++l) xpre[pbuf][l] = load_stream(x + x_off[l] + h * row_units);
-                    const int pr = imin(t2, kP - 1);
+                    const int pr = imin(imax(p0 - kPadY + t2, row_lo), row_hi);
 #pragma unroll
                     for (int l = 0; l < LPTD; ++l) dpre[pbuf][l] = load_stream(dy + d_off[l] + pr * row_units);
                 }
@@ -414,8 +437,8 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                 //    written here are not read in this step, except for dy entries of the weight
                 //    gradient whose filter row is out of range and whose product is ignored.
                 if (t + 1 < ROWS) {
-                    const int hn = t + 1 - kPadY;
-                    if (hn >= 0 && hn < kH) {
+                    const int hn = p0 - 2 * kPadY + t + 1;
+                    if (t + 1 >= kPadY && hn >= 0 && hn < kH) {
 #pragma unroll
                         for (int l = 0; l < LPTX; ++l)
                             if (x_lds[l] >= 0)
@@ -423,7 +446,8 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                                     x_ok[l] ? xpre[(uu + 1) % PF][l] : zero4;
                     }
                     const int dslot = (t + 1) % NRD;
-                    const bool drow_ok = t + 1 < kP;
+                    const int dn = p0 - kPadY + t + 1;
+                    const bool drow_ok = t + 1 < bh_eff + 2 * kPadY && dn >= 0 && dn < kP;
 #pragma unroll
                     for (int l = 0; l < LPTD; ++l)
                         if (d_lds[l] >= 0)
@@ -440,7 +464,7 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
 #pragma unroll
                         for (int m = 0; m < NPAIR; ++m) {
                             const int i2 = tbase - 2 * m;
-                            if (i2 >= 0 && i2 < kP) {
+                            if (i2 + 1 >= own_lo && i2 < own_hi) {
                                 const int d = sp + 2 * m;  // = t - i2
                                 if (d <= kR && x_live) {
 #pragma unroll
@@ -472,12 +496,13 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                     }
                 }
 
-                // 6. the dx row that received its last tap (row t - py): stage it, reset its slot
+                // 6. the dx row that received its last tap (row p0-2py+t): stage it if the block
+                //    owns it, reset its slot
                 {
                     const int slot = pmod(ph - (kR - 1), NS);
                     const int a = slot >> 1;
                     const int j = slot & 1;
-                    const bool emit = hcur >= 0 && hcur < kH;
+                    const bool emit = t >= 2 * kPadY && t < 2 * kPadY + bh_eff;
                     if (wave_active && out_j == j) {
 #pragma unroll
                         for (int i = 0; i < TPW; ++i) {

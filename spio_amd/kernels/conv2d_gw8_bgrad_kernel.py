@@ -30,7 +30,7 @@ MAX_WAVES = 16
 MAX_LDS_BYTES = 128 * 1024
 MAX_LOADS_PER_THREAD = 4
 MAX_REGISTERS = 224  # estimated fragments + accumulators + prefetch buffers, in 32-bit registers
-MAX_GEOMETRIES = 10
+MAX_GEOMETRIES = 12
 PREFETCH_CHOICES = (2, 4)
 
 
@@ -40,6 +40,9 @@ class Conv2dGw8BgradConfig:
 
     Attributes:
         groups: channel groups per workgroup (one wave each, times `split`).
+        block_h: rows of grad_input (and of grad_output for the weight gradient) per
+            workgroup; 0 = the whole image.  Smaller blocks give more workgroups at the price
+            of re-reading the padding rows of grad_output and x at the block borders.
         block_n: images whose rows are laid side by side in one staged row.
         block_n_iters: image blocks a workgroup processes before it publishes grad_weight.
         prefetch: rows of global loads in flight ahead of the computed row (even).
@@ -48,6 +51,7 @@ class Conv2dGw8BgradConfig:
     """
 
     groups: int = 4
+    block_h: int = 0
     block_n: int = 1
     block_n_iters: int = 1
     prefetch: int = 4
@@ -63,6 +67,7 @@ def bgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig) -> Dic
     """Host mirror of the compile-time constants of conv2d_gw8_bgrad_mfma.hip."""
     r, s = params.r, params.s
     gb, nb, iters, ts, pf = config.groups, config.block_n, config.block_n_iters, config.split, config.prefetch
+    bh = config.block_h or params.p
     s2 = 2 * ((s + 1) // 2)
     nblk = s2 // 2
     wpi = params.w + s - 1
@@ -99,10 +104,10 @@ def bgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig) -> Dic
         NBLK=nblk, KC=kc, CPW=cpw, WT=wt, TPW=tpw, THREADS=threads,
         LDS_BYTES=max(stream_bytes, filter_bytes, publish_bytes),
         LPTX=lptx, LPTD=lptd, REGISTERS=registers,
-        GBLKS=divup(params.groups, gb), NBLKS=divup(params.n, nb * iters),
+        BH=bh, GBLKS=divup(params.groups, gb), PBLKS=divup(params.p, bh), NBLKS=divup(params.n, nb * iters),
         PIXEL_EFF=(nb * params.q) / (32.0 * kc),
     )  # fmt: skip
-    g["NUM_BLOCKS"] = g["GBLKS"] * g["NBLKS"]
+    g["NUM_BLOCKS"] = g["GBLKS"] * g["PBLKS"] * g["NBLKS"]
     return g
 
 
@@ -113,6 +118,7 @@ def _config_is_legal(params, config) -> bool:
     return (
         config.groups * config.split <= MAX_WAVES
         and config.split <= min(g["KC"], g["WT"])
+        and 0 <= config.block_h <= params.p
         and config.block_n * config.block_n_iters <= max(params.n, 1)
         and g["LDS_BYTES"] <= MAX_LDS_BYTES
         and g["LPTX"] <= MAX_LOADS_PER_THREAD
@@ -127,7 +133,8 @@ def _score(params, config, num_cus) -> float:
     g = bgrad_geometry(params, config)
     group_eff = params.groups / (g["GBLKS"] * config.groups)
     quant = divup(g["NUM_BLOCKS"], num_cus) * num_cus / g["NUM_BLOCKS"]
-    stream_us = 6.0 * params.n * params.c * params.h * params.w / 5.0e6
+    halo = 1.0 + (2.0 / 3.0) * (2 * params.padding_h if g["PBLKS"] > 1 else 0) / g["BH"]
+    stream_us = halo * 6.0 * params.n * params.c * params.h * params.w / 5.0e6
     publish_us = g["NUM_BLOCKS"] * config.groups * params.r * params.s * 64.0 / (128 * 2.1e3)
     split_line = 1.0 if (config.groups * 16) % 128 == 0 or config.groups == params.groups else 1.12
     return (quant * split_line / (g["PIXEL_EFF"] ** 0.3 * group_eff)) * (1.0 + publish_us / stream_us)
@@ -139,13 +146,16 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None) -> List[Conv2dGw8Bgr
     G = params.groups
     group_choices = sorted({g for g in (4, 8, 16, G) if g <= min(G, MAX_WAVES)}) or [min(G, MAX_WAVES)]
     geometries = []
+    row_choices = [0] + sorted({bh for bh in (7, 14, 28) if bh < params.p}, reverse=True)
     for gb in group_choices:
-        for nb in (1, 2, 4, 8):
-            for iters in (1, 2, 4):
-                for ts in (1, 2):
-                    cfg = Conv2dGw8BgradConfig(groups=gb, block_n=nb, block_n_iters=iters, prefetch=2, split=ts)
-                    if _config_is_legal(params, cfg):
-                        geometries.append((_score(params, cfg, num_cus), cfg))
+        for bh in row_choices:
+            for nb in (1, 2, 4, 8):
+                for iters in (1, 2, 4):
+                    for ts in (1, 2):
+                        cfg = Conv2dGw8BgradConfig(groups=gb, block_h=bh, block_n=nb, block_n_iters=iters,
+                                                   prefetch=2, split=ts)  # fmt: skip
+                        if _config_is_legal(params, cfg):
+                            geometries.append((_score(params, cfg, num_cus), cfg))
     geometries.sort(key=lambda sc: sc[0])
     configs = []
     for _, base in geometries[:MAX_GEOMETRIES]:
@@ -161,7 +171,8 @@ def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig, _dev
     assert _config_is_legal(params, config), f"illegal configuration {config} for {params}"
     g = bgrad_geometry(params, config)
     defines = _shape_defines(params)
-    defines.update(SPIO_GB=config.groups, SPIO_NB=config.block_n, SPIO_ITERS=config.block_n_iters,
+    defines.update(SPIO_GB=config.groups, SPIO_BH=g["BH"], SPIO_NB=config.block_n,
+                   SPIO_ITERS=config.block_n_iters,
                    SPIO_PF=config.prefetch, SPIO_TS=config.split,
                    SPIO_HAS_BIAS=int(params.has_bias))  # fmt: skip
     return KernelSpec(defines, LaunchParams(grid=g["NUM_BLOCKS"], block=g["THREADS"]), SOURCE, notes=g)

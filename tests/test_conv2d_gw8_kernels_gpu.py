@@ -77,7 +77,21 @@ def test_bgrad_explicit_configs():
                           configs=[Conv2dGw8BgradConfig(groups=4, block_n=2, block_n_iters=1, prefetch=2, split=2),
                                    Conv2dGw8BgradConfig(groups=4, block_n=2, block_n_iters=2, prefetch=4, split=1),
                                    Conv2dGw8BgradConfig(groups=6, block_n=2, block_n_iters=1, prefetch=2, split=2),
-                                   Conv2dGw8BgradConfig(groups=4, block_n=4, block_n_iters=1, prefetch=2, split=2)])  # fmt: skip
+                                   Conv2dGw8BgradConfig(groups=4, block_n=4, block_n_iters=1, prefetch=2, split=2),
+                                   # row blocks with halo rows, a last block that is not full (20 = 7+7+6)
+                                   Conv2dGw8BgradConfig(groups=4, block_h=7, block_n=2, block_n_iters=1, prefetch=2, split=1),
+                                   Conv2dGw8BgradConfig(groups=6, block_h=14, block_n=1, block_n_iters=2, prefetch=4, split=1),
+                                   Conv2dGw8BgradConfig(groups=4, block_h=1, block_n=2, block_n_iters=1, prefetch=2, split=1)])  # fmt: skip
+    # 5x5 filter (two halo rows), odd block height, bias
+    params = Conv2dGw8Params(n=3, c=16, h=13, w=18, r=5, s=5, padding=2, has_bias=True)
+    run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params,
+                          configs=[Conv2dGw8BgradConfig(groups=2, block_h=5, block_n=1, block_n_iters=1, prefetch=2, split=1),
+                                   Conv2dGw8BgradConfig(groups=2, block_h=3, block_n=2, block_n_iters=1, prefetch=2, split=2)])  # fmt: skip
+    # one filter row (no halo rows) with a bias: the bias sum's extra step, odd block height
+    params = Conv2dGw8Params(n=2, c=16, h=9, w=11, r=1, s=3, padding=(0, 1), has_bias=True)
+    run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params,
+                          configs=[Conv2dGw8BgradConfig(groups=2, block_h=3, block_n=1, block_n_iters=1, prefetch=2, split=1),
+                                   Conv2dGw8BgradConfig(groups=2, block_h=4, block_n=1, block_n_iters=1, prefetch=2, split=1)])  # fmt: skip
 
 
 def test_bgrad_is_not_offered_when_the_image_size_changes():
