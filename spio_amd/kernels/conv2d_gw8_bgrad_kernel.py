@@ -30,8 +30,7 @@ MAX_WAVES = 16
 MAX_LDS_BYTES = 128 * 1024
 MAX_LOADS_PER_THREAD = 4
 MAX_REGISTERS = 224  # estimated fragments + accumulators + prefetch buffers, in 32-bit registers
-MAX_GEOMETRIES = 12
-PREFETCH_CHOICES = (2, 4)
+GEOMETRIES_PER_HEIGHT = 6
 
 
 @dataclass(frozen=True)
@@ -145,24 +144,25 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None) -> List[Conv2dGw8Bgr
     num_cus = getattr(device_attr, "multiprocessor_count", 256) or 256
     G = params.groups
     group_choices = sorted({g for g in (4, 8, 16, G) if g <= min(G, MAX_WAVES)}) or [min(G, MAX_WAVES)]
-    geometries = []
+    # Rank the geometries of every row-block height separately and keep the best few of each:
+    # whether whole images or row blocks win depends on the shape in ways the score does not
+    # capture (contiguity of the channel block, halo re-reads, workgroups per compute unit).
     row_choices = [0] + sorted({bh for bh in (7, 14, 28) if bh < params.p}, reverse=True)
-    for gb in group_choices:
-        for bh in row_choices:
+    configs = []
+    for bh in row_choices:
+        geometries = []
+        for gb in group_choices:
             for nb in (1, 2, 4, 8):
                 for iters in (1, 2, 4):
                     for ts in (1, 2):
                         cfg = Conv2dGw8BgradConfig(groups=gb, block_h=bh, block_n=nb, block_n_iters=iters,
-                                                   prefetch=2, split=ts)  # fmt: skip
+                                                   prefetch=4, split=ts)  # fmt: skip
                         if _config_is_legal(params, cfg):
                             geometries.append((_score(params, cfg, num_cus), cfg))
-    geometries.sort(key=lambda sc: sc[0])
-    configs = []
-    for _, base in geometries[:MAX_GEOMETRIES]:
-        for pf in PREFETCH_CHOICES:
-            cfg = replace(base, prefetch=pf)
-            if _config_is_legal(params, cfg):
-                configs.append(cfg)
+        geometries.sort(key=lambda sc: sc[0])
+        configs += [cfg for _, cfg in geometries[:GEOMETRIES_PER_HEIGHT]]
+    # a shallower pipeline for the first few: it wins where rows are short
+    configs += [replace(cfg, prefetch=2) for cfg in configs[:GEOMETRIES_PER_HEIGHT]]
     return configs
 
 
