@@ -43,6 +43,7 @@ MEASURED_TRAFFIC_BYTES = {
     ("target", "fprop"): 104_710_000,
     ("target", "dgrad"): 104_720_000,
     ("target", "wgrad"): 105_510_000,
+    ("target", "bgrad"): 163_270_000,
 }
 CACHE_BYTES = 256 * 1024 * 1024
 
