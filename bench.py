@@ -247,9 +247,9 @@ def main():
 
     # The backward half of the step runs the way the product's backward op runs it: one fused
     # data+weight gradient kernel where the recorded times say it beats the two separate ones.
-    from spio_amd.functional.conv2d_gw8_function import _fused_backward_kernel
+    from spio_amd.functional import fused_backward_kernel
 
-    k_fused = _fused_backward_kernel(params, device)
+    k_fused = fused_backward_kernel(params, device)
 
     def step(i):
         s = sets[i % nsets]

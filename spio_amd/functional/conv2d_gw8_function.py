@@ -43,7 +43,7 @@ _fused_choice = {}
 _fused_choice_lock = threading.Lock()
 
 
-def _fused_backward_kernel(params: Conv2dGw8Params, device):
+def fused_backward_kernel(params: Conv2dGw8Params, device):
     """The fused data+weight gradient kernel if it should run for `params`, else None."""
     mode = os.environ.get("SPIO_FUSED_BACKWARD", "auto").strip().lower()
     if mode in ("0", "false", "off", "no") or not bgrad_is_supported(params):
@@ -185,7 +185,7 @@ def conv2d_gw8_backward_op(
 
     grad_bias = None
     grad_input = None
-    fused = _fused_backward_kernel(params, inputs.device) if needs_input_grad and needs_weight_grad else None
+    fused = fused_backward_kernel(params, inputs.device) if needs_input_grad and needs_weight_grad else None
     if fused is not None:
         # one pass over grad_output for both gradients (and grad_bias when the layer has a bias)
         grad_weight = torch.zeros_like(weight, dtype=torch.float32)

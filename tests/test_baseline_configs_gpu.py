@@ -53,6 +53,18 @@ def test_full_size_against_oracle(name):
     oracle.check_close(dw, dw_e, acc_depth=depth[2], what=f"{name} wgrad")
 
 
+def test_target_size_with_separate_backward_kernels(monkeypatch):
+    """The recorded times make the backward op pick the fused kernel at the target size; with
+    fusing switched off the separate data- and weight-gradient kernels must give the same answer."""
+    monkeypatch.setenv("SPIO_FUSED_BACKWARD", "0")
+    params, seed = CONFIGS["target"]
+    x, w, dy, _y, dx, dw = _run(params, seed)
+    depth = Conv2dStats(params, output_names=["grad_input", "grad_weight"]).accumulation_depths
+    dx_e, dw_e, _ = oracle.grads_torch(x, w, None, dy, params.padding_h, params.padding_w)
+    oracle.check_close(dx, dx_e, acc_depth=depth[0], what="target dgrad (separate)")
+    oracle.check_close(dw, dw_e, acc_depth=depth[1], what="target wgrad (separate)")
+
+
 @pytest.mark.parametrize("name", ["cfg2", "cfg3"])
 def test_adjoint_identities_from_gpu_results(name):
     """<conv(x), dy> == <x, dgrad(dy)> == <w, wgrad(x, dy)>, evaluated in fp64 from what the

@@ -133,18 +133,18 @@ def test_backward_op_fused_and_separate_kernels_agree_with_the_oracle(monkeypatc
 
 
 def test_fused_backward_choice(monkeypatch):
-    from spio_amd.functional.conv2d_gw8_function import _fused_backward_kernel
+    from spio_amd.functional import fused_backward_kernel
 
     dev = torch.device("cuda", 0)
     same = Conv2dGw8Params(n=2, c=16, h=8, w=8, padding=1)
     monkeypatch.setenv("SPIO_FUSED_BACKWARD", "0")
-    assert _fused_backward_kernel(same, dev) is None
+    assert fused_backward_kernel(same, dev) is None
     monkeypatch.setenv("SPIO_FUSED_BACKWARD", "1")
-    assert _fused_backward_kernel(same, dev) is not None
-    assert _fused_backward_kernel(Conv2dGw8Params(n=2, c=16, h=8, w=8, padding=0), dev) is None
+    assert fused_backward_kernel(same, dev) is not None
+    assert fused_backward_kernel(Conv2dGw8Params(n=2, c=16, h=8, w=8, padding=0), dev) is None
     # no recorded times for this shape and far fewer workgroups than compute units: separate kernels
     monkeypatch.setenv("SPIO_FUSED_BACKWARD", "auto")
-    assert _fused_backward_kernel(same, dev) is None
+    assert fused_backward_kernel(same, dev) is None
 
 
 def test_wgrad_accumulates_into_its_output():
