@@ -15,6 +15,7 @@ from spio_amd.kernels import (
     KernelKey,
     KernelParamsLogger,
     LaunchParams,
+    conv2d_gw8_bgrad_kernel_factory,
     conv2d_gw8_kernel_factory,
     conv2d_gw8_wgrad_kernel_factory,
     kernel_params_logging_is_enabled,
@@ -74,8 +75,11 @@ def test_kernel_names_follow_the_reference_convention():
 def test_jit_specialisation_of_every_family(params):
     """hipRTC compiles first/last configuration of each family for gfx950 (no GPU needed)."""
     for factory, kw in ((conv2d_gw8_kernel_factory, {}), (conv2d_gw8_kernel_factory, {"igrad": True}),
-                        (conv2d_gw8_wgrad_kernel_factory, {})):  # fmt: skip
+                        (conv2d_gw8_wgrad_kernel_factory, {}), (conv2d_gw8_bgrad_kernel_factory, {})):  # fmt: skip
         configs = list(factory.configs(params, ATTR, **kw))
+        if not configs:  # the fused backward kernel exists for size-preserving shapes only
+            assert factory is conv2d_gw8_bgrad_kernel_factory
+            continue
         for cfg in {configs[0], configs[-1]}:
             kernel = factory.make_kernel(params, cfg, ATTR, **kw)
             kernel.compile()
@@ -83,6 +87,38 @@ def test_jit_specialisation_of_every_family(params):
             assert kernel.kernel_name.encode() in kernel.code
             with pytest.raises(ValueError):
                 kernel.launch()  # not loaded
+
+
+def test_packaged_tuning_records_name_configurations_that_still_exist():
+    """A packaged record whose configuration is no longer a candidate would be ignored and
+    trigger a sweep on first use; keep the records in step with the configuration spaces."""
+    import dataclasses
+    import os
+
+    import spio_amd.kernels as kernels_pkg
+
+    families = {
+        "spio_conv2d_gw8_fprop": (conv2d_gw8_kernel_factory, {}),
+        "spio_conv2d_gw8_dgrad": (conv2d_gw8_kernel_factory, {"igrad": True}),
+        "spio_conv2d_gw8_wgrad": (conv2d_gw8_wgrad_kernel_factory, {}),
+        "spio_conv2d_gw8_bgrad": (conv2d_gw8_bgrad_kernel_factory, {}),
+    }
+    tuned = os.path.join(os.path.dirname(kernels_pkg.__file__), "tuned")
+    checked = 0
+    for fname in os.listdir(tuned):
+        arch, cus = fname[: -len(".json")].rsplit("_", 1)
+        attr = dataclasses.replace(DeviceAttributes(), arch=arch, multiprocessor_count=int(cus[:-2]))
+        with open(os.path.join(tuned, fname), encoding="utf-8") as f:
+            records = json.load(f)
+        for key, record in records.items():
+            name, encoded = key.split("__")
+            factory, kw = families[name]
+            params = Conv2dGw8Params.decode(encoded)
+            config = factory.config_cls(**record["config"])
+            assert config in list(factory.configs(params, attr, **kw)), f"stale record {key}: {config}"
+            assert record["us"] > 0
+            checked += 1
+    assert checked > 0
 
 
 def test_illegal_config_is_rejected():
