@@ -129,3 +129,20 @@ def test_dgrad_sampled(params):
 @pytest.mark.parametrize("params", sample_params(seed=3), ids=lambda p: p.encode())
 def test_wgrad_sampled(params):
     run_grad_kernel_test(conv2d_gw8_wgrad_kernel_factory, params)
+
+
+def _sampled_same_size(seed, count=6):
+    """Seeded draw from the reference's model-derived shapes the fused backward kernel supports."""
+    import random
+
+    from helpers import reference_test_params
+
+    pool = [p for p in reference_test_params(True) + reference_test_params(False)
+            if bgrad_is_supported(p) and list(conv2d_gw8_bgrad_kernel_factory.configs(p))]  # fmt: skip
+    return random.Random(seed).sample(pool, min(count, len(pool)))
+
+
+@pytest.mark.slow
+@pytest.mark.parametrize("params", _sampled_same_size(seed=4), ids=lambda p: p.encode())
+def test_bgrad_sampled(params):
+    run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params)
