@@ -201,6 +201,35 @@ def test_layer_training_step():
     oracle.check_close(layer.bias.grad, db_e, acc_depth=2 * 12 * 12, what="layer db")
 
 
+@pytest.mark.parametrize("mode", ["0", "1"])
+def test_two_layer_training_step(monkeypatch, mode):
+    """Two stacked layers: the second one's backward needs grad_input, grad_weight and grad_bias,
+    which is where the fused backward kernel runs (mode 1) or the separate kernels (mode 0).
+    Gradients of both layers against the same network built from nn.Conv2d in fp32 on the CPU."""
+    monkeypatch.setenv("SPIO_FUSED_BACKWARD", mode)
+    torch.manual_seed(2)
+    c, groups = 48, 6
+    net = nn.Sequential(Conv2dGw8(c, c, 3, padding=1, groups=groups), nn.ReLU(),
+                        Conv2dGw8(c, c, 5, padding=2, groups=groups))  # fmt: skip
+    ref = nn.Sequential(nn.Conv2d(c, c, 3, padding=1, groups=groups), nn.ReLU(),
+                        nn.Conv2d(c, c, 5, padding=2, groups=groups))  # fmt: skip
+    ref.load_state_dict({k: v.half().float() if v.dim() == 4 else v for k, v in net.state_dict().items()})
+    net = net.cuda().to(memory_format=torch.channels_last)
+    x = torch.randn(3, c, 14, 18).half()
+    dy = torch.randn(3, c, 14, 18).half()
+    with torch.autocast(device_type="cuda", dtype=torch.float16):
+        y = net(x.cuda().contiguous(memory_format=torch.channels_last))
+    y.backward(dy.cuda())
+    y_ref = ref(x.float())
+    y_ref.backward(dy.float())
+    # fp16 activations between the layers: compare with a tolerance scaled to the gradients' size
+    for (name, p_gpu), (_n, p_ref) in zip(net.named_parameters(), ref.named_parameters()):
+        got, want = p_gpu.grad.float().cpu(), p_ref.grad
+        assert got.shape == want.shape
+        err = (got - want).abs().max().item()
+        assert err <= 2e-2 + 5e-3 * want.abs().max().item(), f"{name} mode {mode}: max err {err}"
+
+
 def test_opcheck():
     p = Conv2dGw8Params(n=4, c=64, h=16, w=32, padding=1, has_bias=True)
     x, w, b, _ = oracle.make_args(p.n, p.c, p.h, p.w, 3, 3, 1, 1, True, 0)
