@@ -230,6 +230,44 @@ def test_two_layer_training_step(monkeypatch, mode):
         assert err <= 2e-2 + 5e-3 * want.abs().max().item(), f"{name} mode {mode}: max err {err}"
 
 
+@pytest.mark.parametrize("mode", ["0", "1"])
+def test_ops_replay_correctly_from_a_hip_graph(monkeypatch, mode):
+    """Forward and backward ops captured once into a HIP graph, replayed three times on new
+    data with eager work and synchronisations between the replays; every replay must match the
+    oracle (the launches go to the capturing stream and carry no memset nodes)."""
+    monkeypatch.setenv("SPIO_FUSED_BACKWARD", mode)
+    p = Conv2dGw8Params(n=2, c=32, h=12, w=12, padding=1, has_bias=True)
+    x0, w0, b0, dy0 = oracle.make_args(p.n, p.c, p.h, p.w, 3, 3, 1, 1, True, 0)
+    x, w, b, dy = to_gpu(x0), to_gpu(w0), to_gpu(b0), to_gpu(dy0)
+
+    def run():
+        y = conv2d_gw8(x, w, b, 1, 1, 1, 1, p.groups)
+        dx, dw, db = torch.ops.spio.conv2d_gw8_backward(x, w, b, dy, 1, 1, True, True, True)
+        return y, dx, dw, db
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()  # first use outside the capture: kernel compilation and loading
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            outs = run()
+    torch.cuda.current_stream().wait_stream(side)
+    for trial in range(3):
+        xt, wt, bt, dyt = oracle.make_args(p.n, p.c, p.h, p.w, 3, 3, 1, 1, True, 10 + trial)
+        x.copy_(to_gpu(xt)), w.copy_(to_gpu(wt)), b.copy_(to_gpu(bt)), dy.copy_(to_gpu(dyt))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        y_e = oracle.fprop_torch(xt, wt, bt, 1, 1)
+        dx_e, dw_e, db_e = oracle.grads_torch(xt, wt, bt, dyt, 1, 1)
+        what = f"graph replay {trial} mode {mode}"
+        oracle.check_close(outs[0], y_e, acc_depth=72, what=what + " y")
+        oracle.check_close(outs[1], dx_e, acc_depth=72, what=what + " dx")
+        oracle.check_close(outs[2], dw_e, acc_depth=p.n * p.p * p.q, what=what + " dw")
+        oracle.check_close(outs[3], db_e, acc_depth=p.n * p.p * p.q, what=what + " db")
+
+
 def test_opcheck():
     p = Conv2dGw8Params(n=4, c=64, h=16, w=32, padding=1, has_bias=True)
     x, w, b, _ = oracle.make_args(p.n, p.c, p.h, p.w, 3, 3, 1, 1, True, 0)
