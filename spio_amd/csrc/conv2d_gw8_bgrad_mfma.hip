@@ -91,7 +91,10 @@ constexpr int FPD_D = 16 * WT + 4 * KB - 1;            // dy pixels: data-gradie
 constexpr int FPD = FPD_W > FPD_D ? FPD_W : FPD_D;
 constexpr int GSD = FPD + ((9 - FPD % 16) + 16) % 16;  // dy group stride, = 9 mod 16
 constexpr int NRX = 2;                                 // x ring rows
-constexpr int NRD = 2 * ((kR + 2) / 2);                // dy ring rows: even, >= R+1
+// dy ring rows: even, >= R+1; and at least 4 when the bias is summed, because that sum reads the
+// whole row pair (t-1, t) in the step that stages row t+1 (with a one-row filter the weight
+// gradient itself needs only two rows)
+constexpr int NRD = (SPIO_HAS_BIAS && kR == 1) ? 4 : 2 * ((kR + 2) / 2);
 constexpr int XROW_UNITS = GB * GSX;
 constexpr int DROW_UNITS = GB * GSD + ((4 - (GB * GSD) % 16) + 16) % 16;
 constexpr int OSTRIDE = GB * 16 + 16;        // bytes per pixel in the dx output stage

@@ -92,8 +92,10 @@ constexpr int FPD = 32 * KC;
 constexpr int GSD = FPD + ((9 - FPD % 16) + 16) % 16;  // dy group stride
 constexpr int NRX = 2 * RB;                             // x ring rows: the step's rows and the next step's
 // dy ring rows: the aligned row pairs a step multiplies (R+1 rows with one row per step, up to
-// R+2 with two) plus the rows the step writes for the next one; even.
-constexpr int NRD = 2 * ((kR + 2) / 2) + (RB == 2 ? 2 : 0);
+// R+2 with two) plus the rows the step writes for the next one; even.  The bias sum reads the
+// whole pair (t-1, t) in the step that stages row t+1, so it needs four rows even with a one-row
+// filter, whose weight gradient alone gets by with two.
+constexpr int NRD = ((SPIO_HAS_BIAS && kR == 1) ? 4 : 2 * ((kR + 2) / 2)) + (RB == 2 ? 2 : 0);
 constexpr int XROW_UNITS = GB * GSX;
 // dy ring rows are 64 bytes apart modulo the 256-byte bank period, so the two rows of a
 // pair that one transposing read touches fall into different banks.

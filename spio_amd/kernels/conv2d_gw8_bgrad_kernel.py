@@ -82,7 +82,7 @@ def bgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig) -> Dic
     gsx = fpx + ((9 - fpx % 16) + 16) % 16
     fpd = max(params.padding_w + 32 * kc, 16 * wt + 4 * kb - 1)
     gsd = fpd + ((9 - fpd % 16) + 16) % 16
-    nrd = 2 * ((r + 2) // 2)
+    nrd = 4 if (params.has_bias and r == 1) else 2 * ((r + 2) // 2)
     threads = 64 * gb * ts
     ring_units = 2 * gb * gsx + nrd * (gb * gsd + ((4 - (gb * gsd) % 16) + 16) % 16)
     out_row_bytes = 16 * wt * (gb * 16 + 16)

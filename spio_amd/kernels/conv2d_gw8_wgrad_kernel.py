@@ -82,7 +82,7 @@ def wgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig) -> Dic
     gsd = fpd + ((9 - fpd % 16) + 16) % 16
     rb = config.rows
     nrx = 2 * rb
-    nrd = 2 * ((r + 2) // 2) + (2 if rb == 2 else 0)
+    nrd = (4 if (params.has_bias and r == 1) else 2 * ((r + 2) // 2)) + (2 if rb == 2 else 0)
     threads = 64 * gb * ts
     lds_rings = (nrx * gb * gsx + nrd * (gb * gsd + ((4 - (gb * gsd) % 16) + 16) % 16)) * 16
     # the same LDS block holds the reduction scratch at the end: per-wave row-slot halves, the

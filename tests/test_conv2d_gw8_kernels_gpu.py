@@ -34,6 +34,10 @@ SANITY = [
     Conv2dGw8Params(n=5, c=8, h=7, w=7, r=2, s=5, padding=(1, 2), has_bias=True),
     # one filter row with a bias and an odd row count: the fused bias sum needs its extra step
     Conv2dGw8Params(n=3, c=16, h=9, w=11, r=1, s=3, padding=(0, 1), has_bias=True),
+    # one filter row, bias, many rows per image: the bias sum reads a row pair while the next row
+    # is staged, which needs a deeper grad_output ring than the one-row weight gradient itself
+    Conv2dGw8Params(n=1, c=128, h=32, w=32, r=1, s=1, padding=0, has_bias=True),
+    Conv2dGw8Params(n=1, c=128, h=32, w=32, r=1, s=4, padding=(0, 2), has_bias=True),
     # output taller than the input, with a bias: grad_output rows whose x row is all padding
     Conv2dGw8Params(n=2, c=16, h=6, w=6, r=3, s=3, padding=2, has_bias=True),
 ]
