@@ -343,6 +343,14 @@ def main():
             "kernel": k_fused.kernel_name,
             "note": "fused dgrad+wgrad as the backward op runs it for this shape; replaces the "
                     "dgrad and wgrad launches in the timed step",
+            # the same time priced with the bytes the two separate kernels need for this work
+            "unfused_accounting": {
+                "bytes": kernels["dgrad"]["bytes"] + kernels["wgrad"]["bytes"],
+                "GB/s": round((kernels["dgrad"]["bytes"] + kernels["wgrad"]["bytes"]) / (ms * 1e-3) / 1e9, 1),
+                "frac_of_hbm_peak": round(
+                    (kernels["dgrad"]["bytes"] + kernels["wgrad"]["bytes"]) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4
+                ),
+            },
         }
 
     in_step = [n for n in kernels if (n in ("fprop", "bgrad") if k_fused is not None else n != "bgrad")]
