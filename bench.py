@@ -385,6 +385,10 @@ def main():
             "first_use_seconds": round(setup_s, 2),
         },
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+        "value_note": "algorithmic bytes of fprop + dgrad + wgrad (the reference's per-direction accounting) "
+                      "divided by the time of one step as the operators run it"
+                      + ("; the backward half of this step is one fused kernel that reads grad_output once, "
+                         "so the step moves fewer bytes than the numerator counts" if k_fused is not None else ""),
         "hip_graph_replay": None if graph_ms_per_step is None else {
             "ms_per_step": round(graph_ms_per_step, 5),
             "value": round(step_bytes / (graph_ms_per_step * 1e-3) / 1e9, 1),
