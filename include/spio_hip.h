@@ -133,6 +133,28 @@ typedef struct spio_hip_launch_desc {
 int spio_hip_launch_sequence_timed(const spio_hip_launch_desc_t* descs, int stages, int num_sets,
                                    void* stream, int warmup, int iters, float* elapsed_ms);
 
+/* Size of the library's static device workspace (one copy per GPU). */
+#define SPIO_HIP_SCRATCH_BYTES (32u * 1024u * 1024u)
+
+/* Like spio_hip_launch, for kernels that need a workspace in device memory
+ * (the two-stage weight gradient: the main kernel stores per-workgroup partial
+ * sums into it, its `_reduce` kernel reads them back), for callers that cannot
+ * allocate: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  No counterpart in the reference, whose kernels need no
+ * workspace.  Kernel argument number `scratch_param` (a device pointer) is
+ * replaced by the address of a fixed SPIO_HIP_SCRATCH_BYTES array that lives
+ * in the library's own device code, of which the kernel may use the first
+ * `scratch_bytes`; more than SPIO_HIP_SCRATCH_BYTES is rejected with
+ * SPIO_HIP_ERR_ARGUMENT.  The call allocates and frees nothing.  Every call on
+ * one GPU shares that GPU's array: it keeps the last call's contents, and
+ * calls that overlap on one GPU (different streams or threads) race on it. */
+int spio_hip_launch_scratch(void* function,
+                            unsigned grid_x, unsigned grid_y, unsigned grid_z,
+                            unsigned block_x, unsigned block_y, unsigned block_z,
+                            unsigned dynamic_lds_bytes, void* stream,
+                            void** params, int num_params,
+                            int scratch_param, size_t scratch_bytes);
+
 /* Asynchronous fill of a device buffer with zero bytes on `stream`; used for
  * the pre-zeroed weight-gradient contract
  * (spio/functional/conv2d_gw8_function.py:124-127) by callers without torch. */

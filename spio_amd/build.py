@@ -1,8 +1,11 @@
 """Builds the native pieces of the package in-tree.
 
-`build_native()` compiles csrc/spio_hip.cpp into csrc/libspio_hip.so with the
-host C++ compiler.  The library has no link-time dependency on the HIP
-runtime (it binds it with dlopen), so it builds on machines without a GPU.
+`build_native()` builds csrc/libspio_hip.so from csrc/spio_hip.cpp (host C++;
+it binds the HIP runtime and hipRTC with dlopen) and csrc/spio_hip_scratch.hip
+(hipcc, gfx950: the static device workspace and the launch that uses it, which
+links the HIP runtime by its soname, so the copy a host framework has already
+mapped is the one used).  hipcc cross-compiles, so this builds on machines
+without a GPU.
 
 `check_kernels()` compiles every HIP kernel source for gfx950 with hipcc for
 a list of representative shape specialisations; at run time the same sources
@@ -39,26 +42,45 @@ def _include_dir() -> str:
     return CSRC_DIR
 
 
-def build_native(force: bool = True, verbose: bool = False) -> str:
-    """Compile libspio_hip.so; returns its path."""
-    src = os.path.join(CSRC_DIR, "spio_hip.cpp")
-    if not force and os.path.exists(LIB_PATH) and os.path.getmtime(LIB_PATH) >= os.path.getmtime(src):
-        return LIB_PATH
-    cxx = os.environ.get("CXX") or shutil.which("g++") or shutil.which("c++")
-    if cxx is None:
-        raise RuntimeError("no host C++ compiler found to build libspio_hip.so")
-    tmp = LIB_PATH + f".tmp{os.getpid()}"
-    cmd = [
-        cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall",
-        f"-I{_include_dir()}", f"-I{os.path.join(ROCM_HOME, 'include')}",
-        "-o", tmp, src, "-ldl", "-lpthread",
-    ]  # fmt: skip
+def _run(cmd, what, verbose=False):
     if verbose:
         print(" ".join(cmd))
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
-        raise RuntimeError(f"building libspio_hip.so failed:\n{proc.stdout}\n{proc.stderr}")
-    os.replace(tmp, LIB_PATH)
+        raise RuntimeError(f"{what} failed:\n{' '.join(cmd)}\n{proc.stdout}\n{proc.stderr}")
+
+
+def build_native(force: bool = True, verbose: bool = False) -> str:
+    """Compile libspio_hip.so; returns its path."""
+    host_src = os.path.join(CSRC_DIR, "spio_hip.cpp")
+    dev_src = os.path.join(CSRC_DIR, "spio_hip_scratch.hip")
+    deps = [host_src, dev_src, os.path.join(CSRC_DIR, "spio_hip_internal.h"),
+            os.path.join(_include_dir(), "spio_hip.h")]  # fmt: skip
+    if not force and os.path.exists(LIB_PATH) and all(
+        os.path.getmtime(LIB_PATH) >= os.path.getmtime(d) for d in deps
+    ):
+        return LIB_PATH
+    cxx = os.environ.get("CXX") or shutil.which("g++") or shutil.which("c++")
+    if cxx is None:
+        raise RuntimeError("no host C++ compiler found to build libspio_hip.so")
+    hipcc = shutil.which("hipcc") or os.path.join(ROCM_HOME, "bin", "hipcc")
+    includes = [f"-I{_include_dir()}", f"-I{CSRC_DIR}", f"-I{os.path.join(ROCM_HOME, 'include')}"]
+    tag = f".tmp{os.getpid()}"
+    host_obj = os.path.join(CSRC_DIR, f"spio_hip{tag}.o")
+    dev_obj = os.path.join(CSRC_DIR, f"spio_hip_scratch{tag}.o")
+    tmp = LIB_PATH + tag
+    try:
+        _run([cxx, "-O2", "-std=c++17", "-fPIC", "-Wall", "-fvisibility-inlines-hidden", *includes,
+              "-c", "-o", host_obj, host_src], "compiling spio_hip.cpp", verbose)  # fmt: skip
+        _run([hipcc, *HIPCC_DEVICE_FLAGS, "-fPIC", *includes, "-c", "-o", dev_obj, dev_src],
+             "compiling spio_hip_scratch.hip", verbose)  # fmt: skip
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, host_obj, dev_obj,
+              "-ldl", "-lpthread"], "linking libspio_hip.so", verbose)  # fmt: skip
+        os.replace(tmp, LIB_PATH)
+    finally:
+        for f in (host_obj, dev_obj, tmp):
+            if os.path.exists(f):
+                os.remove(f)
     return LIB_PATH
 
 

@@ -9,6 +9,7 @@
 // for the launches issued here.
 
 #include "spio_hip.h"
+#include "spio_hip_internal.h"
 
 #include <dlfcn.h>
 
@@ -305,8 +306,15 @@ int spio_hip_func_set_max_dynamic_lds(void* function, int bytes) {
     return SPIO_HIP_OK;
 }
 
-static int check_launch_args(void* function, unsigned gx, unsigned gy, unsigned gz, unsigned bx,
-                             unsigned by, unsigned bz, int num_params) {
+}  // extern "C"
+
+int spio_hip_set_error(int code, const char* text) {
+    g_last_error = text ? text : "";
+    return code;
+}
+
+int spio_hip_check_launch_args(void* function, unsigned gx, unsigned gy, unsigned gz, unsigned bx,
+                               unsigned by, unsigned bz, int num_params) {
     if (!function) return fail(SPIO_HIP_ERR_ARGUMENT, "launch: null function handle");
     if (num_params < 0 || num_params > 16)
         return fail(SPIO_HIP_ERR_ARGUMENT, "launch: %d kernel arguments, at most 16 are supported",
@@ -320,11 +328,13 @@ static int check_launch_args(void* function, unsigned gx, unsigned gy, unsigned 
     return SPIO_HIP_OK;
 }
 
+extern "C" {
+
 int spio_hip_launch(void* function, unsigned grid_x, unsigned grid_y, unsigned grid_z,
                     unsigned block_x, unsigned block_y, unsigned block_z,
                     unsigned dynamic_lds_bytes, void* stream, void** params, int num_params) {
     REQUIRE_READY();
-    int rc = check_launch_args(function, grid_x, grid_y, grid_z, block_x, block_y, block_z,
+    int rc = spio_hip_check_launch_args(function, grid_x, grid_y, grid_z, block_x, block_y, block_z,
                                num_params);
     if (rc) return rc;
     if (num_params > 0 && !params) return fail(SPIO_HIP_ERR_ARGUMENT, "launch: null params");
@@ -340,7 +350,7 @@ int spio_hip_launch_timed(void* function, unsigned grid_x, unsigned grid_y, unsi
                           int num_sets, int num_params, int warmup, int iters,
                           float* elapsed_ms) {
     REQUIRE_READY();
-    int rc = check_launch_args(function, grid_x, grid_y, grid_z, block_x, block_y, block_z,
+    int rc = spio_hip_check_launch_args(function, grid_x, grid_y, grid_z, block_x, block_y, block_z,
                                num_params);
     if (rc) return rc;
     if (!param_sets || num_sets < 1 || warmup < 0 || iters < 1 || !elapsed_ms)
@@ -384,7 +394,7 @@ int spio_hip_launch_sequence_timed(const spio_hip_launch_desc_t* descs, int stag
         return fail(SPIO_HIP_ERR_ARGUMENT, "spio_hip_launch_sequence_timed: bad argument");
     for (int i = 0; i < stages * num_sets; ++i) {
         const spio_hip_launch_desc_t& d = descs[i];
-        int rc = check_launch_args(d.function, d.grid[0], d.grid[1], d.grid[2], d.block[0],
+        int rc = spio_hip_check_launch_args(d.function, d.grid[0], d.grid[1], d.grid[2], d.block[0],
                                    d.block[1], d.block[2], d.num_params);
         if (rc) return rc;
         if (d.num_params > 0 && !d.params)

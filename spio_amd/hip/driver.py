@@ -90,6 +90,10 @@ _SIGNATURES = {
         [_vp] + [ctypes.c_uint] * 7 + [_vp, ctypes.POINTER(_vp), ctypes.c_int],
         ctypes.c_int,
     ),
+    "spio_hip_launch_scratch": (
+        [_vp] + [ctypes.c_uint] * 7 + [_vp, ctypes.POINTER(_vp), ctypes.c_int, ctypes.c_int, ctypes.c_size_t],
+        ctypes.c_int,
+    ),
     "spio_hip_launch_timed": (
         [_vp] + [ctypes.c_uint] * 7
         + [_vp, ctypes.POINTER(ctypes.POINTER(_vp)), ctypes.c_int, ctypes.c_int, ctypes.c_int,
@@ -111,6 +115,9 @@ _SIGNATURES = {
     "spio_hip_runtime_version": ([ctypes.POINTER(ctypes.c_int)], ctypes.c_int),
     "spio_hiprtc_version": ([ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)], ctypes.c_int),
 }  # fmt: skip
+
+# Size of the library's static device workspace (SPIO_HIP_SCRATCH_BYTES in spio_hip.h).
+SCRATCH_BYTES = 32 * 1024 * 1024
 
 _lib = None
 _lib_lock = threading.Lock()
@@ -314,6 +321,21 @@ class Function:
         rc = _lib.spio_hip_launch(
             self._handle, grid[0], grid[1], grid[2], block[0], block[1], block[2],
             shared_mem_bytes, stream or None, params, len(args),
+        )  # fmt: skip
+        if rc:
+            _check(rc)
+
+    def launch_scratch(self, grid, block, args, scratch_param: int, scratch_bytes: int,
+                       shared_mem_bytes: int = 0, stream: int = 0):  # fmt: skip
+        """Launch with the library's static device workspace as argument `scratch_param`.
+
+        Nothing is allocated; `args[scratch_param]` is ignored (pass None).  All calls on one
+        GPU share the workspace, so launches that overlap on one GPU must not both use it.
+        """
+        params, _values = self.marshal(args)
+        rc = _lib.spio_hip_launch_scratch(
+            self._handle, grid[0], grid[1], grid[2], block[0], block[1], block[2],
+            shared_mem_bytes, stream or None, params, len(args), int(scratch_param), int(scratch_bytes),
         )  # fmt: skip
         if rc:
             _check(rc)

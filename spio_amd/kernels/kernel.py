@@ -115,8 +115,14 @@ class Kernel:
             raise ValueError("kernel arguments must be GPU tensors")
         return device
 
-    def launch(self, *args):
-        """Asynchronous launch on torch's current stream of the arguments' device."""
+    def launch(self, *args, static_workspace: bool = False):
+        """Asynchronous launch on torch's current stream of the arguments' device.
+
+        `static_workspace=True` makes a two-stage kernel take its workspace from the native
+        library's fixed device array instead of torch's allocator (for callers that must not
+        allocate); it raises when the kernel needs more than that array holds, and launches that
+        overlap on one GPU must not both use it.
+        """
         try:
             device = self._prepare(args)
             spec = self.kernel_spec
@@ -124,6 +130,13 @@ class Kernel:
             stream = torch.cuda.current_stream(device).cuda_stream
             if self.epilogue_function is None:
                 self.function.launch(lp.grid, lp.block, args, lp.shared_mem_bytes, stream)
+            elif static_workspace:
+                ep = spec.epilogue_launch_params
+                nbytes = spec.workspace_bytes
+                self.function.launch_scratch(lp.grid, lp.block, (None,) + args[1:], 0, nbytes,
+                                             lp.shared_mem_bytes, stream)  # fmt: skip
+                self.epilogue_function.launch_scratch(ep.grid, ep.block, (args[0], None), 1, nbytes,
+                                                      ep.shared_mem_bytes, stream)  # fmt: skip
             else:
                 workspace = self._workspace(device)
                 self.function.launch(lp.grid, lp.block, (workspace,) + args[1:], lp.shared_mem_bytes, stream)
