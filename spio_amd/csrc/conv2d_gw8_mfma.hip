@@ -31,6 +31,16 @@
 //     pixel-major order and stored with one coalesced 16-byte store per lane.
 //   * One workgroup barrier per step; global loads run SPIO_PF rows ahead of
 //     the row being computed.
+//   * Global memory is reached through buffer instructions whose hardware
+//     bounds check does the predication: lanes without data carry an
+//     out-of-range offset, rows outside the image use a descriptor of size
+//     zero.  Such loads return zeros (the zero padding of the convolution) and
+//     such stores are dropped, so no memory instruction sits under a branch.
+//     Together with the fully unrolled step loop this lets the compiler count
+//     the outstanding loads and stores exactly: the wait before a row is used
+//     is for that row only.  (A wait counter covers loads and stores alike; a
+//     count merged over paths that issue different numbers of them degrades
+//     to the smallest, i.e. to waiting for rows that are not needed yet.)
 #include "spio_conv_common.h"
 
 using namespace spio;
@@ -49,6 +59,9 @@ using namespace spio;
 #endif
 #ifndef SPIO_NB
 #define SPIO_NB 1
+#endif
+#ifndef SPIO_XCD_CHUNK
+#define SPIO_XCD_CHUNK 0
 #endif
 
 namespace {
@@ -80,7 +93,8 @@ constexpr int TPW = (WT + TS - 1) / TS;     // tiles per wave
 constexpr int FP = 16 * WT + 4 * KB - 1;    // pixels any fragment read can touch
 constexpr int GS = FP + ((9 - FP % 16) + 16) % 16;  // group stride in pixels, = 9 mod 16
 constexpr int NR = 2;                               // ring rows
-constexpr int RING_ROW_UNITS = GB * GS;             // 16-byte units per ring row
+constexpr int RING_ROW_UNITS = GB * GS + 1;         // 16-byte units per ring row (+1: dump cell)
+constexpr int DUMP_UNIT = GB * GS;                  // where lanes without a cell write
 constexpr int OSTRIDE = GB * 16 + 16;               // bytes per pixel in the output stage
 constexpr int OUT_ROW_BYTES = 16 * WT * OSTRIDE;
 constexpr int IN_CELLS = F * GB;
@@ -94,13 +108,28 @@ constexpr int NUM_BLOCKS = GBLKS * PBLKS * NBLKS;
 constexpr int STEPS = BP + kR - 1;
 
 constexpr int gcd_(int a, int b) { return b == 0 ? a : gcd_(b, a % b); }
-constexpr int UNROLL = NS / gcd_(NS, PF) * PF;  // lcm(NS, PF); even, so also a multiple of NR
+constexpr int LCM = NS / gcd_(NS, PF) * PF;  // lcm(NS, PF); even, so also a multiple of NR
+// Up to SPIO_MAX_UNROLL steps the whole step loop is unrolled (every rotation index and every
+// "is there a row to load / to store" is then a compile-time fact); longer loops run in chunks
+// of lcm(NS, PF) steps.
+#ifndef SPIO_MAX_UNROLL
+#define SPIO_MAX_UNROLL 64
+#endif
+constexpr bool kFullUnroll = STEPS <= SPIO_MAX_UNROLL;
+constexpr int CHUNK = kFullUnroll ? (STEPS + LCM - 1) / LCM * LCM : LCM;
 
-static_assert(PF >= 2 && WAVES <= 16 && UNROLL % NR == 0, "bad configuration");
+static_assert(PF >= 2 && WAVES <= 16 && LCM % NR == 0, "bad configuration");
 constexpr int STREAM_UNITS = NR * RING_ROW_UNITS + 2 * OUT_ROW_BYTES / 16;
 constexpr int FILTER_UNITS = kIgrad ? GB * 8 * kR * kS : 0;  // staged filters (data gradient only)
 constexpr int LDS_UNITS = STREAM_UNITS > FILTER_UNITS ? STREAM_UNITS : FILTER_UNITS;
 static_assert(LDS_UNITS * 16 <= 160 * 1024, "LDS overflow");
+
+// Byte extents of the NB-image block a workgroup addresses through one buffer descriptor.
+constexpr long long SRC_IMAGE_BYTES = (long long)SH * SW * kC * 2;
+constexpr long long DST_IMAGE_BYTES = (long long)DH * DW * kC * 2;
+static_assert(NB * SRC_IMAGE_BYTES < (1ll << 31) && NB * DST_IMAGE_BYTES < (1ll << 31),
+              "an image block must stay below 2 GiB (32-bit buffer offsets)");
+constexpr unsigned OOB = 0x80000000u;  // offset of a lane without data: beyond every descriptor
 
 constexpr int pmod(int a, int m) { return ((a % m) + m) % m; }
 
@@ -111,9 +140,11 @@ constexpr int pmod(int a, int m) { return ((a % m) + m) % m; }
 #ifndef SPIO_HALO_CACHED
 #define SPIO_HALO_CACHED 0
 #endif
-SPIO_DEVICE spio_uint4 load_row(const spio_uint4* p, int step) {
-    if (SPIO_HALO_CACHED && (step < kR - 1 || step >= BP)) return *p;
-    return load_stream(p);
+constexpr int AUX_NT = SPIO_NT ? 2 : 0;  // cache-policy operand of the buffer instructions
+
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+SPIO_DEVICE rsrc_t make_rsrc(const void* base, int bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
 }
 
 }  // namespace
@@ -124,100 +155,172 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
     // One LDS block: the source-row ring, then the two output-stage rows.  The data-gradient
     // mode first uses the same block to stage the filters of the workgroup's groups.
     __shared__ spio_uint4 lds[LDS_UNITS];
-    spio_uint4* const ring = lds;
-    unsigned char* const ostage = reinterpret_cast<unsigned char*>(lds + NR * RING_ROW_UNITS);
+    // pointers typed in the LDS address space: 32-bit address arithmetic, constant parts of an
+    // index end up in the instruction's offset field
+    typedef __attribute__((address_space(3))) spio_uint4* lds_u4p;
+    typedef __attribute__((address_space(3))) unsigned char* lds_bytep;
+    const lds_u4p ring = (lds_u4p)lds;
+    const lds_bytep ostage = (lds_bytep)(ring + NR * RING_ROW_UNITS);
 
     const int tid = thread_id();
     const int lane = tid & 63;
-    // the wave index as a scalar: conditions on it become scalar branches, so that no MFMA
-    // (which ignores the lane mask) is ever issued under an empty mask
+    // the wave index as a scalar: whatever depends on it alone stays in scalar registers
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wg = wave % GB;  // group within the workgroup
     const int ws = wave / GB;  // tile split index
 
     // Workgroup -> (image block, channel block, row block), row block fastest.
-    // Consecutive workgroup ids are dealt round-robin to the 8 XCDs; remap so
-    // that each XCD works on a contiguous range of tiles (neighbouring row
-    // blocks share halo rows through that XCD's L2).
+    // Consecutive workgroup ids are dealt round-robin to the 8 XCDs.  Remap so that runs of
+    // SPIO_XCD_CHUNK consecutive tiles land on one XCD (neighbouring row blocks share halo rows
+    // through that XCD's L2) while the tiles in flight on the whole device at any moment still
+    // form one compact, advancing range of addresses (HBM streams best through such a front;
+    // eight distant fronts, one per XCD, cost several per cent).  0 = one contiguous range of
+    // tiles per XCD.
     int b = block_id();
-    if (NUM_BLOCKS % 8 == 0) b = (b & 7) * (NUM_BLOCKS / 8) + (b >> 3);
+    {
+        constexpr int CH = SPIO_XCD_CHUNK;
+        if (CH == 0) {
+            if (NUM_BLOCKS % 8 == 0) b = (b & 7) * (NUM_BLOCKS / 8) + (b >> 3);
+        } else if (CH > 1 && NUM_BLOCKS % (8 * CH) == 0) {
+            const int x = b & 7;   // XCD
+            const int k = b >> 3;  // position in that XCD's sequence
+            b = (k / CH) * (8 * CH) + x * CH + k % CH;
+        }
+    }
     const int pb = b % PBLKS;
     const int cb = (b / PBLKS) % GBLKS;
     const int nb = b / (PBLKS * GBLKS);
     const int p0 = pb * BP;
     const int n0 = nb * NB;
     const int gglob = cb * GB + wg;
-    const bool wave_active = gglob < kGroups;
+    const bool wave_active = gglob < kGroups;  // idle waves compute on zeros and store nothing
+
+    // ---- buffer descriptors: the workgroup's image block of src and of dst ----
+    // Offsets are relative to the block's first image; images past the end of the batch lie
+    // beyond the descriptor's size, so their loads give zeros and their stores are dropped.
+    const int images = imin(NB, kN - n0);
+    const rsrc_t rs_src = make_rsrc(reinterpret_cast<const unsigned char*>(src) + n0 * SRC_IMAGE_BYTES,
+                                    (int)(images * SRC_IMAGE_BYTES));
+    const rsrc_t rs_dst = make_rsrc(reinterpret_cast<const unsigned char*>(dst) + n0 * DST_IMAGE_BYTES,
+                                    (int)(images * DST_IMAGE_BYTES));
+    const rsrc_t rs_src_none = make_rsrc(reinterpret_cast<const unsigned char*>(src), 0);
+    const rsrc_t rs_dst_none = make_rsrc(reinterpret_cast<const unsigned char*>(dst), 0);
 
     // ---- loop-invariant addressing of the cooperative row load ----
-    // Every thread issues the same number of loads on every step, without branches, so that the
-    // compiler can count outstanding loads exactly and wait only for the row it needs (a load
-    // under a branch makes it wait for all of them).  Cells that hold no source data (halo
-    // columns, missing images or groups) load a valid dummy address and are zeroed when the row
-    // is written to LDS.
-    int in_off[LPT];   // 16-byte units from src; row term excluded
-    bool in_ok[LPT];   // the cell carries source data
-    int in_lds[LPT];   // 16-byte unit inside a ring row; -1 = no cell
-    const int dummy_off = n0 * SH * SW * kGroups;  // first unit of the workgroup's first image
+    // Every thread issues the same loads on every step.  Cells that hold no source data (halo
+    // columns, missing groups) carry the out-of-range offset: the load returns zeros, which is
+    // what the halo must hold.  Threads without a cell write to the row's dump cell.
+    unsigned in_voff[LPT];  // byte offset inside the image block; row term excluded
+    int in_lds[LPT];        // 16-byte unit inside a ring row
 #pragma unroll
     for (int l = 0; l < LPT; ++l) {
         const int cell = tid + THREADS * l;
-        in_off[l] = dummy_off;
-        in_ok[l] = false;
-        in_lds[l] = -1;
+        in_voff[l] = OOB;
+        in_lds[l] = DUMP_UNIT;
         if (cell < IN_CELLS) {
             const int g = cell % GB;
             const int f = cell / GB;
             const int img = f / WPI;
             const int col = f % WPI - EPX;
             in_lds[l] = g * GS + f;
-            if (col >= 0 && col < SW && n0 + img < kN && cb * GB + g < kGroups) {
-                in_off[l] = ((n0 + img) * SH * SW + col) * kGroups + cb * GB + g;
-                in_ok[l] = true;
-            }
+            if (col >= 0 && col < SW && cb * GB + g < kGroups)
+                in_voff[l] = (unsigned)(((img * SH * SW + col) * kGroups + cb * GB + g) * 16);
         }
     }
-    const long long row_units = (long long)SW * kGroups;  // 16-byte units per source row
-    const long long dst_row_units = (long long)DW * kGroups;
+    constexpr int SRC_ROW_BYTES = SW * kC * 2;
+    constexpr int DST_ROW_BYTES = DW * kC * 2;
 
-    // ---- rows 0..PF-1 into registers, first of all: their latency covers the filter set-up ----
+    // Source row `t` of this workgroup (image row p0 + t - EPY) for every cell of the thread.
+    // Rows outside the image read through the empty descriptor: zeros, the vertical padding.
+    auto load_row = [&](spio_uint4(&regs)[LPT], int t) {
+        const int h = p0 + t - EPY;
+        const bool inside = h >= 0 && h < SH;
+        const rsrc_t rs = inside ? rs_src : rs_src_none;
+        // (readfirstlane: the row offset must stay in a scalar register whatever the optimiser
+        //  makes of the clamp)
+        const int soff = __builtin_amdgcn_readfirstlane(imin(imax(h, 0), SH - 1) * SRC_ROW_BYTES);
+        const bool halo = t < kR - 1 || t >= BP;
+#pragma unroll
+        for (int l = 0; l < LPT; ++l) {
+            Pack16 v;
+            v.i = (SPIO_HALO_CACHED && halo)
+                      ? __builtin_amdgcn_raw_buffer_load_b128(rs, (int)in_voff[l], soff, 0)
+                      : __builtin_amdgcn_raw_buffer_load_b128(rs, (int)in_voff[l], soff, AUX_NT);
+            regs[l] = v.u;
+        }
+    };
+
+    // ---- filter loads, first of all ----
+    // Loads of one wave return in order, so what is requested first is what the first
+    // multiplication waits for: the filters (a few loads per lane) go ahead of the PF source
+    // rows, and the first step can start as soon as source row 0 has landed.  Branch-free: dead
+    // taps and idle waves load a valid address and are zeroed when the fragments are built.
+    constexpr int WLPT = kIgrad ? (GB * 8 * kR * kS + THREADS - 1) / THREADS : NS * KB;
+    spio_uint4 wraw[WLPT];
+    if (!kIgrad) {
+        // A[m = out channel ch][c] = w[8g+ch][r][s][c]: 16 contiguous bytes per lane.
+        // Lane (m = lane%16, kb = lane/16): row slot j = m/8, channel m%8, column tap 4u+kb;
+        // the filter row of slot j at distance d is r = (d - j) mod NS (none if r >= R).
+        const int m = lane & 15;
+        const int kb = lane >> 4;
+        const int j = m >> 3;
+        const int ch = m & 7;
+        const int gsafe = wave_active ? gglob : 0;
+#pragma unroll
+        for (int d = 0; d < NS; ++d) {
+#pragma unroll
+            for (int u = 0; u < KB; ++u) {
+                const int r = (d - j + NS) % NS;
+                const int s = 4 * u + kb;
+                const int rr = r < kR ? r : 0;
+                const int ss = s < kS ? s : 0;
+                wraw[d * KB + u] = *reinterpret_cast<const spio_uint4*>(
+                    weights + (((long long)(8 * gsafe + ch) * kR + rr) * kS + ss) * 8);
+            }
+        }
+    } else {
+        // the workgroup's filters as they lie in memory ([group][jj][r][s][8 ch]), WLPT units per thread
+        constexpr int WUNITS = GB * 8 * kR * kS;
+#pragma unroll
+        for (int l = 0; l < WLPT; ++l) {
+            const int i = imin(tid + THREADS * l, WUNITS - 1);
+            const int g = i / (8 * kR * kS);
+            const int rem = i % (8 * kR * kS);
+            const int gs = cb * GB + g < kGroups ? cb * GB + g : 0;
+            wraw[l] = reinterpret_cast<const spio_uint4*>(weights)[(long long)gs * (8 * kR * kS) + rem];
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);  // keep the filter loads ahead of the row loads
+
+    // ---- rows 0..PF-1 into registers: their latency covers the rest of the set-up ----
     spio_uint4 pre[PF][LPT];
 #pragma unroll
-    for (int t = 0; t < PF; ++t) {
-        // rows outside the image are loaded from the nearest real row and never used
-        const int h = imin(imax(p0 + t - EPY, 0), SH - 1);
-#pragma unroll
-        for (int l = 0; l < LPT; ++l) pre[t][l] = load_row(src + in_off[l] + h * row_units, t);
-    }
+    for (int t = 0; t < PF; ++t) load_row(pre[t], imin(t, STEPS - 1));
+    __builtin_amdgcn_sched_barrier(0);  // ... and the row loads ahead of everything that waits
 
     // ---- loop-invariant addressing of the cooperative row store ----
-    int out_off[SPT];  // 16-byte units from dst; row term excluded; -1 = nothing to store
-    int out_lds[SPT];  // byte offset inside an output-stage row
+    unsigned out_voff[SPT];  // byte offset inside the image block; row term excluded
+    int out_lds[SPT];        // byte offset inside an output-stage row
 #pragma unroll
     for (int s = 0; s < SPT; ++s) {
         const int cell = tid + THREADS * s;
-        out_off[s] = -1;
+        out_voff[s] = OOB;
         out_lds[s] = 0;
         if (cell < OUT_CELLS) {
             const int g = cell % GB;
             const int q = (cell / GB) % DW;
             const int img = cell / (GB * DW);
             out_lds[s] = (img * WPI + q) * OSTRIDE + g * 16;
-            if (n0 + img < kN && cb * GB + g < kGroups)
-                out_off[s] = ((n0 + img) * DH * DW + q) * kGroups + cb * GB + g;
+            if (cb * GB + g < kGroups) out_voff[s] = (unsigned)(((img * DH * DW + q) * kGroups + cb * GB + g) * 16);
         }
     }
 
     // ---- filter fragments: wfrag[d][u], d = (phase - 2*acc) mod NS ----
-    // Lane (m = lane%16, kb = lane/16): row slot j = m/8, channel m%8, column tap 4u+kb;
-    // the filter row of slot j at distance d is r = (d - j) mod NS (none if r >= R).
     spio_half8 wfrag[NS][KB];
     if (!kIgrad) {
-        // A[m = out channel ch][c] = w[8g+ch][r][s][c]: 16 contiguous bytes per lane.
         const int m = lane & 15;
         const int kb = lane >> 4;
         const int j = m >> 3;
-        const int ch = m & 7;
 #pragma unroll
         for (int d = 0; d < NS; ++d) {
 #pragma unroll
@@ -225,10 +328,7 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
                 const int r = (d - j + NS) % NS;
                 const int s = 4 * u + kb;
                 Pack16 v;
-                v.u = spio_uint4{0u, 0u, 0u, 0u};
-                if (wave_active && r < kR && s < kS)
-                    v.u = *reinterpret_cast<const spio_uint4*>(
-                        weights + (((long long)(8 * gglob + ch) * kR + r) * kS + s) * 8);
+                v.u = (r < kR && s < kS) ? wraw[d * KB + u] : spio_uint4{0u, 0u, 0u, 0u};
                 wfrag[d][u] = v.h;
             }
         }
@@ -239,14 +339,11 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
         // in a 16-lane block source lane 4*jr+t supplies 4 channels (half t%2) of row jj = jr for
         // the row slot t/2, and result lane i receives rows jj = 0..3 of column i = 8*slot + ch.
         constexpr int WUNITS = GB * 8 * kR * kS;
-        spio_uint4* wlds = lds;  // ring and output stage are not in use yet
-        for (int i = tid; i < WUNITS; i += THREADS) {
-            const int g = i / (8 * kR * kS);
-            const int rem = i % (8 * kR * kS);
-            spio_uint4 v = spio_uint4{0u, 0u, 0u, 0u};
-            if (cb * GB + g < kGroups)
-                v = reinterpret_cast<const spio_uint4*>(weights)[(long long)(cb * GB + g) * (8 * kR * kS) + rem];
-            wlds[i] = v;
+        const lds_u4p wlds = ring;  // ring and output stage are not in use yet
+#pragma unroll
+        for (int l = 0; l < WLPT; ++l) {
+            const int i = tid + THREADS * l;
+            if (i < WUNITS) wlds[i] = wraw[l];
         }
         block_sync();
         const int kb = lane >> 4;
@@ -265,15 +362,14 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
                 // clamp the address of dead taps; their result is discarded below
                 const int rr = r_src < kR ? kR - 1 - r_src : 0;
                 const int ss = s < kS ? kS - 1 - s : 0;
-                const unsigned char* base = reinterpret_cast<const unsigned char*>(wlds) +
-                                            ((((wg * 8 + jr) * kR + rr) * kS + ss) * 16) + (t4 & 1) * 8;
+                const lds_bytep base = (lds_bytep)wlds + ((((wg * 8 + jr) * kR + rr) * kS + ss) * 16) + (t4 & 1) * 8;
                 union {
                     spio_short4 q[2];
                     spio_half8 h;
                 } v;
                 v.q[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)base);
                 v.q[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(base + 4 * kR * kS * 16));
-                if (!(wave_active && r_mine < kR && s < kS)) v.h = spio_half8{0, 0, 0, 0, 0, 0, 0, 0};
+                if (!(r_mine < kR && s < kS)) v.h = spio_half8{0, 0, 0, 0, 0, 0, 0, 0};
                 wfrag[d][u] = v.h;
             }
         }
@@ -285,6 +381,9 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
     const int out_j = lane >> 5;
     const int out_kh = (lane >> 4) & 1;
     const int out_n = lane & 15;
+    // this lane's place in a staged output row (tile 0 of the wave) and in a ring row
+    const lds_bytep ostage_lane = ostage + (16 * ws + out_n) * OSTRIDE + wg * 16 + out_kh * 8;
+    const int frag_unit = wg * GS + (lane & 15) + (lane >> 4);
     float bias_reg[4] = {0.f, 0.f, 0.f, 0.f};
     if (kHasBias && wave_active) {
 #pragma unroll
@@ -297,68 +396,73 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
         for (int a = 0; a < NACC; ++a)
             acc[i][a] = spio_float4{bias_reg[0], bias_reg[1], bias_reg[2], bias_reg[3]};
 
-    // ---- zero the ring once: halo and slack cells are never written again ----
-    for (int i = tid; i < NR * RING_ROW_UNITS; i += THREADS) ring[i] = spio_uint4{0u, 0u, 0u, 0u};
-
+    // ---- zero the slack cells behind each group's pixels once: fragment reads of the last
+    //      tiles touch them (they meet zero filter taps, so they must be finite), nothing ever
+    //      writes them ----
+    {
+        constexpr int SLACK = GS - F;
+        for (int i = tid; i < NR * GB * SLACK; i += THREADS) {
+            const int row = i / (GB * SLACK);
+            const int g = (i / SLACK) % GB;
+            ring[row * RING_ROW_UNITS + g * GS + F + i % SLACK] = spio_uint4{0u, 0u, 0u, 0u};
+        }
+    }
 
     // ---- row 0 into the ring ----
     block_sync();  // ring zeroed
-    {
-        const int h = p0 - EPY;
-        if (h >= 0 && h < SH) {
 #pragma unroll
-            for (int l = 0; l < LPT; ++l)
-                if (in_lds[l] >= 0) ring[in_lds[l]] = in_ok[l] ? pre[0][l] : spio_uint4{0u, 0u, 0u, 0u};
-        }
-    }
+    for (int l = 0; l < LPT; ++l) ring[in_lds[l]] = pre[0][l];
     block_sync();
 
     // Coalesced store of the output row staged at step `ts` (in stage buffer `obuf`): the row
-    // that received its last tap at that step.  Called one step later, after the barrier.
+    // that received its last tap at that step.  Called one step later, after the barrier.  Steps
+    // that finish no row, and rows past the end of the image, store through the empty
+    // descriptor: the instructions are issued all the same and the hardware drops them.
     auto store_output_row = [&](int ts, int obuf) {
         const int p = p0 + ts - (kR - 1);
-        if (ts >= kR - 1 && p < DH) {
+        const bool real = ts >= kR - 1 && p < DH;
+        const rsrc_t rs = real ? rs_dst : rs_dst_none;
+        const int soff = __builtin_amdgcn_readfirstlane(imin(imax(p, 0), DH - 1) * DST_ROW_BYTES);
 #pragma unroll
-            for (int s = 0; s < SPT; ++s) {
-                if (out_off[s] >= 0) {
-                    const spio_uint4 v =
-                        *reinterpret_cast<const spio_uint4*>(ostage + obuf * OUT_ROW_BYTES + out_lds[s]);
-                    store_stream(v, dst + out_off[s] + p * dst_row_units);
-                }
-            }
+        for (int s = 0; s < SPT; ++s) {
+            Pack16 v;
+            v.u = *(lds_u4p)(ostage + obuf * OUT_ROW_BYTES + out_lds[s]);
+            __builtin_amdgcn_raw_buffer_store_b128(v.i, rs, (int)out_voff[s], soff, AUX_NT);
         }
     };
 
-    for (int tb = 0; tb < STEPS; tb += UNROLL) {
+    for (int tb = 0; tb < STEPS; tb += CHUNK) {
 #pragma unroll
-        for (int uu = 0; uu < UNROLL; ++uu) {
+        for (int uu = 0; uu < CHUNK; ++uu) {
             const int t = tb + uu;
             if (t >= STEPS) break;
-            constexpr int kDummy = 0;
-            (void)kDummy;
             const int ph = uu % NS;        // compile-time after unrolling
             const int rbuf = uu % NR;      // ring row holding source row t
             const int obuf = uu & 1;       // output stage buffer of this step
             const int pbuf = uu % PF;      // register buffer that held row t
 
-            // 1. prefetch source row t+PF (its register buffer is free: row t is in LDS)
-            {
-                const int tt = t + PF;
-                if (PF < STEPS) {  // compile-time: with PF >= STEPS the prologue loaded every row
-                    // past the last row the loads repeat it (cache hits) and are never used
-                    const int h = imin(imax(p0 + imin(tt, STEPS - 1) - EPY, 0), SH - 1);
+            // 1. prefetch source row t+PF (its register buffer is free: row t is in LDS).  Past the
+            //    last row the chunked loop still issues its loads (through the empty descriptor), so
+            //    that every step has the same number of them; the unrolled loop leaves them out.
+            if (PF < STEPS && (!kFullUnroll || t + PF < STEPS)) {
+                if (t + PF < STEPS) {
+                    load_row(pre[pbuf], t + PF);
+                } else {
 #pragma unroll
-                    for (int l = 0; l < LPT; ++l) pre[pbuf][l] = load_row(src + in_off[l] + h * row_units, tt);
+                    for (int l = 0; l < LPT; ++l) {
+                        Pack16 v;
+                        v.i = __builtin_amdgcn_raw_buffer_load_b128(rs_src_none, (int)in_voff[l], 0, 0);
+                        pre[pbuf][l] = v.u;
+                    }
                 }
             }
 
             // 2. multiply source row t into the live output rows.  The fragment reads are issued
-            //    first; the previous step's output row is stored while they are in flight.
-            const int hcur = p0 + t - EPY;
-            const bool row_live = wave_active && hcur >= 0 && hcur < SH;
+            //    first; the previous step's output row is stored while they are in flight.  Rows
+            //    above and below the image are rows of zeros in the ring: no special case.
             spio_half8 bfrag[TPW][KB];
-            if (row_live) {
-                const spio_uint4* rrow = ring + rbuf * RING_ROW_UNITS + wg * GS + (lane & 15) + (lane >> 4);
+            {
+                const lds_u4p rrow = ring + rbuf * RING_ROW_UNITS + frag_unit;
 #pragma unroll
                 for (int i = 0; i < TPW; ++i) {
                     const int tile = ws + TS * i;
@@ -366,26 +470,24 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
 #pragma unroll
                         for (int u = 0; u < KB; ++u) {
                             Pack16 v;
-                            v.u = rrow[16 * tile + 4 * u];
+                            v.u = rrow[16 * TS * i + 16 * ws + 4 * u];
                             bfrag[i][u] = v.h;
                         }
                     }
                 }
             }
-            store_output_row(t - 1, (uu + 1) & 1);
-            if (row_live) {
+            if (!kFullUnroll || t >= kR) store_output_row(t - 1, (uu + 1) & 1);
 #pragma unroll
-                for (int i = 0; i < TPW; ++i) {
-                    const int tile = ws + TS * i;
-                    if (TS == 1 || tile < WT) {
+            for (int i = 0; i < TPW; ++i) {
+                const int tile = ws + TS * i;
+                if (TS == 1 || tile < WT) {
 #pragma unroll
-                        for (int a = 0; a < NACC; ++a) {
-                            const int d = pmod(ph - 2 * a, NS);
+                    for (int a = 0; a < NACC; ++a) {
+                        const int d = pmod(ph - 2 * a, NS);
 #pragma unroll
-                            for (int u = 0; u < KB; ++u)
-                                acc[i][a] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                                    wfrag[d][u], bfrag[i][u], acc[i][a], 0, 0, 0);
-                        }
+                        for (int u = 0; u < KB; ++u)
+                            acc[i][a] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                wfrag[d][u], bfrag[i][u], acc[i][a], 0, 0, 0);
                     }
                 }
             }
@@ -396,7 +498,7 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
                 const int a = slot >> 1;
                 const int j = slot & 1;
                 const bool emit = t >= kR - 1;
-                if (wave_active && out_j == j) {
+                if (out_j == j) {
 #pragma unroll
                     for (int i = 0; i < TPW; ++i) {
                         const int tile = ws + TS * i;
@@ -405,9 +507,8 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
                                 Pack8 o;
 #pragma unroll
                                 for (int e = 0; e < 4; ++e) o.h[e] = (spio_half)acc[i][a][e];
-                                *reinterpret_cast<spio_uint2*>(ostage + obuf * OUT_ROW_BYTES +
-                                                               (16 * tile + out_n) * OSTRIDE +
-                                                               wg * 16 + out_kh * 8) = o.u;
+                                typedef __attribute__((address_space(3))) spio_uint2* lds_u2p;
+                                *(lds_u2p)(ostage_lane + obuf * OUT_ROW_BYTES + 16 * TS * i * OSTRIDE) = o.u;
                             }
 #pragma unroll
                             for (int e = 0; e < 4; ++e) acc[i][a][e] = bias_reg[e];
@@ -417,19 +518,13 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
             }
 
             // 4. source row t+1 (loaded earlier) into the other ring row
-            {
-                const int hn = p0 + t + 1 - EPY;
-                if (t + 1 < STEPS && hn >= 0 && hn < SH) {
+            if (t + 1 < STEPS) {
 #pragma unroll
-                    for (int l = 0; l < LPT; ++l)
-                        if (in_lds[l] >= 0)
-                            ring[((uu + 1) % NR) * RING_ROW_UNITS + in_lds[l]] =
-                                in_ok[l] ? pre[(uu + 1) % PF][l] : spio_uint4{0u, 0u, 0u, 0u};
-                }
+                for (int l = 0; l < LPT; ++l)
+                    ring[((uu + 1) % NR) * RING_ROW_UNITS + in_lds[l]] = pre[(uu + 1) % PF][l];
             }
 
             block_sync();
-
         }
     }
     store_output_row(STEPS - 1, (STEPS - 1) & 1);  // the last row

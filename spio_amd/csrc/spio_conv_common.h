@@ -92,6 +92,7 @@ SPIO_DEVICE void atomic_add_f32(float* address, float value) {
 // Bit-cast helpers between the 16-byte vector views of one (pixel, group).
 union Pack16 {
     spio_uint4 u;
+    spio_uint4 i;  // the buffer builtins' 128-bit operand type
     spio_half8 h;
     spio_half4 h4[2];
 };

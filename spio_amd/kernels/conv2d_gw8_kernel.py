@@ -7,7 +7,7 @@ padding (R-1-py, S-1-px), :73-83).  The tile configuration is re-designed for
 CDNA4: see csrc/conv2d_gw8_mfma.hip for what the fields mean on the device.
 """
 
-from dataclasses import dataclass
+from dataclasses import dataclass, replace
 from math import gcd
 from typing import Dict, List
 
@@ -24,11 +24,13 @@ MFMA_SOURCE = "conv2d_gw8_mfma.hip"
 DIRECT_SOURCE = "conv2d_gw8_direct.hip"
 
 MAX_WAVES = 16
-MAX_LDS_BYTES = 64 * 1024
+MAX_LDS_BYTES = 128 * 1024
+MAX_UNROLLED_STEPS = 64  # SPIO_MAX_UNROLL of the kernel: up to here the step loop is fully unrolled
 MAX_LOADS_PER_THREAD = 8
 MAX_ACCUMULATORS = 16
 MAX_CONFIGS = 32
-PREFETCH_CHOICES = (2, 4, 8, 16)
+PREFETCH_CHOICES = (2, 4, 8, 12, 16)
+MAX_GEOMETRIES = 24  # tile geometries that enter the sweep; the best few also try the other cache/XCD policies
 
 
 @dataclass(frozen=True)
@@ -44,6 +46,9 @@ class Conv2dGw8Config:
         nontemporal: 1 = stream activations with the non-temporal hint.
         halo_cached: 1 = load rows shared with neighbouring row blocks with the default
             cache policy so the second reader can hit in L2.
+        xcd_chunk: consecutive tiles that go to the same XCD (they share halo rows through its
+            L2) before the next run of tiles goes to the next XCD; 0 = one contiguous range of
+            tiles per XCD, 1 = tiles dealt round-robin.
         variant: "mfma" (row-streaming MFMA kernel) or "direct" (one thread per
             output pixel-group; any shape).
     """
@@ -55,7 +60,8 @@ class Conv2dGw8Config:
     prefetch: int = 2
     variant: str = "mfma"
     nontemporal: int = 1
-    halo_cached: int = 0
+    halo_cached: int = 1
+    xcd_chunk: int = 4
 
 
 def direction_geometry(params: Conv2dGw8Params, igrad: bool) -> Dict[str, int]:
@@ -81,7 +87,7 @@ def mfma_geometry(params: Conv2dGw8Params, config: Conv2dGw8Config, igrad: bool)
     gs = fp + ((9 - fp % 16) + 16) % 16
     threads = 64 * gb * ts
     ostride = gb * 16 + 16
-    lds = 2 * gb * gs * 16 + 2 * 16 * wt * ostride
+    lds = 2 * (gb * gs + 1) * 16 + 2 * 16 * wt * ostride  # ring rows (+ dump cell) and two output-stage rows
     if igrad:  # the data gradient stages its groups' filters in the same block first
         lds = max(lds, gb * 8 * r * s * 16)
     d.update(
@@ -106,7 +112,10 @@ def _mfma_config_is_legal(params, config, igrad) -> bool:
         and g["LPT"] <= MAX_LOADS_PER_THREAD
         and g["TPW"] * g["NACC"] <= MAX_ACCUMULATORS
         and config.prefetch >= 2
-        and g["UNROLL"] <= 16
+        # longer loops run in chunks of lcm(row slots, prefetch) steps: keep those chunks small
+        and (g["STEPS"] <= MAX_UNROLLED_STEPS or g["UNROLL"] <= 16)
+        # 32-bit buffer offsets inside a workgroup's image block
+        and config.block_n * params.c * max(params.h * params.w, params.p * params.q) * 2 < 2**31
         and g["LPT"] * config.prefetch <= 24
     )
 
@@ -140,7 +149,9 @@ def _mfma_score(params, config, igrad, num_cus: int) -> float:
     big_block = 1.08 if g["THREADS"] > 512 else 1.0
     # a workgroup that covers only part of a 128-byte line of a pixel shares it with another one
     split_line = 1.0 if (config.groups * 16) % 128 == 0 or config.groups == params.groups else 1.12
-    return traffic * quant * starve * few_waves * big_block * split_line / (tile_eff ** 0.3 * group_eff)
+    # every row block runs block_p steps, also the last, partly empty one
+    ragged = g["PBLKS"] * config.block_p / g["DH"]
+    return traffic * quant * ragged * starve * few_waves * big_block * split_line / (tile_eff ** 0.3 * group_eff)
 
 
 def _get_configs(params: Conv2dGw8Params, device_attr=None, igrad: bool = False) -> List[Conv2dGw8Config]:
@@ -163,7 +174,13 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None, igrad: bool = False)
                         if _mfma_config_is_legal(params, cfg, igrad):
                             found.append((_mfma_score(params, cfg, igrad, num_cus), cfg))
     found.sort(key=lambda sc: sc[0])
-    configs = [cfg for _, cfg in found[:MAX_CONFIGS]]
+    configs = [cfg for _, cfg in found[:MAX_GEOMETRIES]]
+    # the memory-system policies, which the score cannot rank: halo rows with or without the
+    # non-temporal hint, and how tiles are dealt to the XCDs
+    for cfg in list(configs[:4]):
+        for hc, ch in ((0, 4), (1, 0), (0, 0)):
+            configs.append(replace(cfg, halo_cached=hc, xcd_chunk=ch))
+    configs = configs[:MAX_CONFIGS]
     configs.append(Conv2dGw8Config(groups=1, block_p=1, block_n=1, split=1, variant="direct"))
     return configs
 
@@ -197,6 +214,7 @@ def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8Config, _device_a
         SPIO_GB=config.groups, SPIO_BP=config.block_p, SPIO_NB=config.block_n,
         SPIO_TS=config.split, SPIO_PF=config.prefetch,
         SPIO_NT=config.nontemporal, SPIO_HALO_CACHED=config.halo_cached,
+        SPIO_XCD_CHUNK=config.xcd_chunk,
     )  # fmt: skip
     return KernelSpec(
         defines, LaunchParams(grid=g["NUM_BLOCKS"], block=g["THREADS"]), MFMA_SOURCE, notes=g
