@@ -32,7 +32,12 @@
 //     place as a source pixel of the data gradient and, shifted by px, its place opposite x in
 //     the weight gradient;
 //   * publishing of dw (and db) as in the weight-gradient kernel: sums staged in LDS in
-//     grad_weight order, atomics of 64 consecutive floats.
+//     grad_weight order, atomics of 64 consecutive floats;
+//   * global memory through buffer instructions with the hardware bounds check as predicate
+//     (lanes without data: out-of-range offset; rows the block does not need: empty descriptor;
+//     such loads return zeros, such stores are dropped) and a fully unrolled step loop, so that
+//     no memory instruction sits under a branch and the compiler's count of outstanding loads and
+//     stores is exact (see conv2d_gw8_mfma.hip).
 #include "spio_conv_common.h"
 
 using namespace spio;
@@ -51,6 +56,15 @@ using namespace spio;
 #endif
 #ifndef SPIO_HAS_BIAS
 #define SPIO_HAS_BIAS 0
+#endif
+#ifndef SPIO_XCD_CHUNK
+#define SPIO_XCD_CHUNK 0
+#endif
+#ifndef SPIO_HALO_CACHED
+#define SPIO_HALO_CACHED 1
+#endif
+#ifndef SPIO_MAX_UNROLL
+#define SPIO_MAX_UNROLL 40  // a step of this kernel is long: beyond this the unroller gives up
 #endif
 
 namespace {
@@ -95,8 +109,12 @@ constexpr int NRX = 2;                                 // x ring rows
 // whole row pair (t-1, t) in the step that stages row t+1 (with a one-row filter the weight
 // gradient itself needs only two rows)
 constexpr int NRD = (SPIO_HAS_BIAS && kR == 1) ? 4 : 2 * ((kR + 2) / 2);
-constexpr int XROW_UNITS = GB * GSX;
-constexpr int DROW_UNITS = GB * GSD + ((4 - (GB * GSD) % 16) + 16) % 16;
+// ring rows carry one spare unit behind the last group: the cell that threads without a source
+// cell write their (zero) load result to
+constexpr int XROW_UNITS = GB * GSX + 1;
+constexpr int DROW_UNITS = GB * GSD + 1 + ((4 - (GB * GSD + 1) % 16) + 16) % 16;
+constexpr int XDUMP = GB * GSX;
+constexpr int DDUMP = GB * GSD;
 constexpr int OSTRIDE = GB * 16 + 16;        // bytes per pixel in the dx output stage
 constexpr int OUT_ROW_BYTES = 16 * WT * OSTRIDE;
 constexpr int X_CELLS = F * GB;
@@ -113,7 +131,10 @@ constexpr int NUM_BLOCKS = GBLKS * PBLKS * NBLKS;
 constexpr int ROWS = BH + 3 * kPadY + (SPIO_HAS_BIAS && kR == 1 ? 1 : 0);
 
 constexpr int gcd_(int a, int b) { return b == 0 ? a : gcd_(b, a % b); }
-constexpr int UNROLL = NS / gcd_(NS, PF) * PF;  // lcm(NS, PF): even
+constexpr int LCM = NS / gcd_(NS, PF) * PF;  // lcm(NS, PF): even
+// up to SPIO_MAX_UNROLL steps the step loop is unrolled completely, longer ones run in chunks
+constexpr bool kFullUnroll = ROWS <= SPIO_MAX_UNROLL;
+constexpr int UNROLL = kFullUnroll ? (ROWS + LCM - 1) / LCM * LCM : LCM;
 constexpr int pmod(int a, int m) { return ((a % m) + m) % m; }
 
 constexpr int RING_UNITS = NRX * XROW_UNITS + NRD * DROW_UNITS;
@@ -128,6 +149,17 @@ constexpr int max3(int a, int b, int c) { return a > b ? (a > c ? a : c) : (b > 
 constexpr int LDS_UNITS = max3(STREAM_UNITS, FILTER_UNITS, (PUBLISH_FLOATS + 3) / 4);
 static_assert(LDS_UNITS * 16 <= 160 * 1024, "LDS overflow");
 static_assert(PF >= 2 && PF % 2 == 0 && WAVES <= 16, "bad configuration");
+
+constexpr long long IMAGE_BYTES = (long long)kH * kW * kC * 2;  // of x, dy and dx alike
+static_assert(NB * IMAGE_BYTES < (1ll << 31), "an image block must stay below 2 GiB (32-bit buffer offsets)");
+constexpr int ROW_BYTES = kW * kC * 2;
+constexpr unsigned OOB = 0x80000000u;  // offset of a lane without data: beyond every descriptor
+constexpr int AUX_NT = SPIO_NT ? 2 : 0;
+
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+SPIO_DEVICE rsrc_t make_rsrc(const void* base, int bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
 
 SPIO_DEVICE spio_half8 read_tr_pair(const unsigned char* lo, const unsigned char* hi) {
     typedef spio_short4 __attribute__((address_space(3))) * lds_ptr;
@@ -165,8 +197,20 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
     const int wg = wave % GB;
     const int ws = wave / GB;
 
+    // Workgroup ids are dealt round-robin to the 8 XCDs: runs of SPIO_XCD_CHUNK consecutive tiles
+    // go to one XCD (row blocks share halo rows through its L2) while the tiles in flight on the
+    // device form one compact range of addresses; 0 = one contiguous range of tiles per XCD.
     int b = block_id();
-    if (NUM_BLOCKS % 8 == 0) b = (b & 7) * (NUM_BLOCKS / 8) + (b >> 3);
+    {
+        constexpr int CH = SPIO_XCD_CHUNK;
+        if (CH == 0) {
+            if (NUM_BLOCKS % 8 == 0) b = (b & 7) * (NUM_BLOCKS / 8) + (b >> 3);
+        } else if (CH > 1 && NUM_BLOCKS % (8 * CH) == 0) {
+            const int x8 = b & 7;
+            const int k = b >> 3;
+            b = (k / CH) * (8 * CH) + x8 * CH + k % CH;
+        }
+    }
     const int pb = b % PBLKS;
     const int cb = (b / PBLKS) % GBLKS;
     const int nbk = b / (PBLKS * GBLKS);
@@ -248,45 +292,50 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
     const spio_half8 ones8 = spio_half8{1, 1, 1, 1, 1, 1, 1, 1};
     (void)ones8;
 
-    const long long row_units = (long long)kW * kGroups;  // 16-byte units per row of x, dy and dx
     const spio_uint4 zero4 = spio_uint4{0u, 0u, 0u, 0u};
+    const rsrc_t rs_none = make_rsrc(x, 0);  // nothing is in range: loads give zeros, stores vanish
 
     for (int it = 0; it < ITERS; ++it) {
         const int n0 = (nbk * ITERS + it) * NB;
         if (n0 >= kN) break;
 
-        // ---- loop-invariant addressing for this image block (branch-free loads: cells without
-        //      data load a valid address and become zero when written to LDS) ----
-        int x_off[LPTX], x_lds[LPTX];
-        bool x_ok[LPTX];
-        const int dummy = n0 * kH * kW * kGroups;
+        // ---- buffer descriptors of this image block; images past the end of the batch lie
+        //      beyond their size ----
+        const int images = imin(NB, kN - n0);
+        const rsrc_t rs_x = make_rsrc(reinterpret_cast<const unsigned char*>(x) + n0 * IMAGE_BYTES,
+                                      (int)(images * IMAGE_BYTES));
+        const rsrc_t rs_dy = make_rsrc(reinterpret_cast<const unsigned char*>(dy) + n0 * IMAGE_BYTES,
+                                       (int)(images * IMAGE_BYTES));
+        const rsrc_t rs_dx = make_rsrc(reinterpret_cast<const unsigned char*>(grad_input) + n0 * IMAGE_BYTES,
+                                       (int)(images * IMAGE_BYTES));
+
+        // ---- loop-invariant addressing (cells without data carry the out-of-range offset: they
+        //      load zeros, which is what halo and gap cells must hold) ----
+        unsigned x_voff[LPTX];
+        int x_lds[LPTX];
 #pragma unroll
         for (int l = 0; l < LPTX; ++l) {
             const int cell = tid + THREADS * l;
-            x_off[l] = dummy;
-            x_ok[l] = false;
-            x_lds[l] = -1;
+            x_voff[l] = OOB;
+            x_lds[l] = XDUMP;
             if (cell < X_CELLS) {
                 const int g = cell % GB;
                 const int f = cell / GB;
                 const int img = f / WPI;
                 const int col = f % WPI - kPadX;
                 x_lds[l] = g * GSX + f;
-                if (col >= 0 && col < kW && n0 + img < kN && cb * GB + g < kGroups) {
-                    x_off[l] = ((n0 + img) * kH * kW + col) * kGroups + cb * GB + g;
-                    x_ok[l] = true;
-                }
+                if (col >= 0 && col < kW && cb * GB + g < kGroups)
+                    x_voff[l] = (unsigned)(((img * kH * kW + col) * kGroups + cb * GB + g) * 16);
             }
         }
-        // dy cells, and the dx cells of the same (image, column, group): same global offset
-        int d_off[LPTD], d_lds[LPTD], o_lds[LPTD];
-        bool d_ok[LPTD];
+        // dy cells, and the dx cells of the same (image, column, group): same offset
+        unsigned d_voff[LPTD];
+        int d_lds[LPTD], o_lds[LPTD];
 #pragma unroll
         for (int l = 0; l < LPTD; ++l) {
             const int cell = tid + THREADS * l;
-            d_off[l] = dummy;
-            d_ok[l] = false;
-            d_lds[l] = -1;
+            d_voff[l] = OOB;
+            d_lds[l] = DDUMP;
             o_lds[l] = 0;
             if (cell < D_CELLS) {
                 const int g = cell % GB;
@@ -294,40 +343,53 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                 const int img = cell / (GB * kQ);
                 d_lds[l] = g * GSD + img * WPI + q + kPadX;
                 o_lds[l] = (img * WPI + q) * OSTRIDE + g * 16;
-                if (n0 + img < kN && cb * GB + g < kGroups) {
-                    d_off[l] = ((n0 + img) * kP * kQ + q) * kGroups + cb * GB + g;
-                    d_ok[l] = true;
-                }
+                if (cb * GB + g < kGroups)
+                    d_voff[l] = (unsigned)(((img * kP * kQ + q) * kGroups + cb * GB + g) * 16);
             }
         }
+
+        // Rows `t` of x (image row p0-2py+t) and of dy (p0-py+t) for every cell of the thread.
+        // Rows the block does not need read through the empty descriptor (zeros, no traffic).
+        auto load_rows = [&](spio_uint4(&xr)[LPTX], spio_uint4(&dr)[LPTD], int t) {
+            const int h = p0 - 2 * kPadY + t;
+            const rsrc_t rx = (h >= row_lo && h <= row_hi) ? rs_x : rs_none;
+            const int sx = __builtin_amdgcn_readfirstlane(imin(imax(h, 0), kH - 1) * ROW_BYTES);
+            const bool xhalo = h < p0 || h >= p0 + bh_eff;
+#pragma unroll
+            for (int l = 0; l < LPTX; ++l) {
+                Pack16 v;
+                v.i = (SPIO_HALO_CACHED && xhalo) ? __builtin_amdgcn_raw_buffer_load_b128(rx, (int)x_voff[l], sx, 0)
+                                                  : __builtin_amdgcn_raw_buffer_load_b128(rx, (int)x_voff[l], sx, AUX_NT);
+                xr[l] = v.u;
+            }
+            const int pr = p0 - kPadY + t;
+            const rsrc_t rd = (pr >= row_lo && pr <= row_hi) ? rs_dy : rs_none;
+            const int sd = __builtin_amdgcn_readfirstlane(imin(imax(pr, 0), kP - 1) * ROW_BYTES);
+            const bool dhalo = pr < p0 || pr >= p0 + bh_eff;
+#pragma unroll
+            for (int l = 0; l < LPTD; ++l) {
+                Pack16 v;
+                v.i = (SPIO_HALO_CACHED && dhalo) ? __builtin_amdgcn_raw_buffer_load_b128(rd, (int)d_voff[l], sd, 0)
+                                                  : __builtin_amdgcn_raw_buffer_load_b128(rd, (int)d_voff[l], sd, AUX_NT);
+                dr[l] = v.u;
+            }
+        };
 
         // ---- prologue: rows 0..PF-1 into registers ----
         spio_uint4 xpre[PF][LPTX], dpre[PF][LPTD];
 #pragma unroll
-        for (int t = 0; t < PF; ++t) {
-            const int h = imin(imax(p0 - 2 * kPadY + t, row_lo), row_hi);
-#pragma unroll
-            for (int l = 0; l < LPTX; ++l) xpre[t][l] = load_stream(x + x_off[l] + h * row_units);
-            const int pr = imin(imax(p0 - kPadY + t, row_lo), row_hi);
-#pragma unroll
-            for (int l = 0; l < LPTD; ++l) dpre[t][l] = load_stream(dy + d_off[l] + pr * row_units);
-        }
+        for (int t = 0; t < PF; ++t) load_rows(xpre[t], dpre[t], t);
+        __builtin_amdgcn_sched_barrier(0);  // the first loads are on their way before anything waits
         if (it == 0) {
-            // zero both rings once, while the first loads are in flight: halo, gap and slack
-            // cells are never written again
+            // zero both rings once, while the first loads are in flight: the slack cells behind
+            // each group's pixels are never written
             for (int i = tid; i < RING_UNITS; i += THREADS) lds[i] = zero4;
         }
         block_sync();  // rings zeroed / previous image block finished
-        {
-            const bool xrow_ok = kPadY == 0;    // step 0: x row p0 - 2py, needed only without padding
-            const bool drow_ok = p0 - kPadY >= 0;  // step 0: dy row p0 - py
 #pragma unroll
-            for (int l = 0; l < LPTX; ++l)
-                if (x_lds[l] >= 0) xring[x_lds[l]] = (xrow_ok && x_ok[l]) ? xpre[0][l] : zero4;
+        for (int l = 0; l < LPTX; ++l) xring[x_lds[l]] = xpre[0][l];
 #pragma unroll
-            for (int l = 0; l < LPTD; ++l)
-                if (d_lds[l] >= 0) dring[d_lds[l]] = (drow_ok && d_ok[l]) ? dpre[0][l] : zero4;
-        }
+        for (int l = 0; l < LPTD; ++l) dring[d_lds[l]] = dpre[0][l];
         block_sync();
 
         spio_float4 dacc[TPW][NACC];  // data gradient: rotating row slots
@@ -337,17 +399,18 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
             for (int a = 0; a < NACC; ++a) dacc[i][a] = spio_float4{0.f, 0.f, 0.f, 0.f};
 
         // Coalesced store of the dx row staged at step `ts` (row p0 - 2py + ts), one step later.
+        // Steps that finish no row of the block store through the empty descriptor: the
+        // instructions are issued all the same and the hardware drops them.
         auto store_dx_row = [&](int ts, int obuf) {
             const int h = p0 - 2 * kPadY + ts;
-            if (ts >= 2 * kPadY && ts < 2 * kPadY + bh_eff) {
+            const bool real = ts >= 2 * kPadY && ts < 2 * kPadY + bh_eff;
+            const rsrc_t rs = real ? rs_dx : rs_none;
+            const int soff = __builtin_amdgcn_readfirstlane(imin(imax(h, 0), kH - 1) * ROW_BYTES);
 #pragma unroll
-                for (int l = 0; l < LPTD; ++l) {
-                    if (d_ok[l]) {
-                        const spio_uint4 v =
-                            *reinterpret_cast<const spio_uint4*>(ostage + obuf * OUT_ROW_BYTES + o_lds[l]);
-                        store_stream(v, grad_input + d_off[l] + h * row_units);
-                    }
-                }
+            for (int l = 0; l < LPTD; ++l) {
+                Pack16 v;
+                v.u = *reinterpret_cast<const spio_uint4*>(ostage + obuf * OUT_ROW_BYTES + o_lds[l]);
+                __builtin_amdgcn_raw_buffer_store_b128(v.i, rs, (int)d_voff[l], soff, AUX_NT);
             }
         };
 
@@ -422,40 +485,24 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                     }
                 }
 
-                // 2. prefetch rows t+PF (rows past the end repeat a real row and are never used)
-                {
-                    const int t2 = t + PF;
-                    const int h = imin(imax(p0 - 2 * kPadY + t2, row_lo), row_hi);
-#pragma unroll
-                    for (int l = 0; l < LPTX; ++l) xpre[pbuf][l] = load_stream(x + x_off[l] + h * row_units);
-                    const int pr = imin(imax(p0 - kPadY + t2, row_lo), row_hi);
-#pragma unroll
-                    for (int l = 0; l < LPTD; ++l) dpre[pbuf][l] = load_stream(dy + d_off[l] + pr * row_units);
-                }
+                // 2. prefetch rows t+PF.  Rows past the end read through the empty descriptor in the
+                //    chunked loop (every step then issues the same loads); the unrolled loop leaves
+                //    them out.
+                if (!kFullUnroll || t + PF < ROWS) load_rows(xpre[pbuf], dpre[pbuf], t + PF);
 
                 // 3. the dx row finished in the previous step goes out
-                store_dx_row(t - 1, (uu + 1) & 1);
+                if (!kFullUnroll || t - 1 >= 2 * kPadY) store_dx_row(t - 1, (uu + 1) & 1);
 
                 // 4. rows t+1 into LDS (dy rows past the last one become zero).  The ring rows
                 //    written here are not read in this step, except for dy entries of the weight
                 //    gradient whose filter row is out of range and whose product is ignored.
                 if (t + 1 < ROWS) {
-                    const int hn = p0 - 2 * kPadY + t + 1;
-                    if (t + 1 >= kPadY && hn >= 0 && hn < kH) {
 #pragma unroll
-                        for (int l = 0; l < LPTX; ++l)
-                            if (x_lds[l] >= 0)
-                                xring[((sp + 1) & 1) * XROW_UNITS + x_lds[l]] =
-                                    x_ok[l] ? xpre[(uu + 1) % PF][l] : zero4;
-                    }
+                    for (int l = 0; l < LPTX; ++l)
+                        xring[((sp + 1) & 1) * XROW_UNITS + x_lds[l]] = xpre[(uu + 1) % PF][l];
                     const int dslot = (t + 1) % NRD;
-                    const int dn = p0 - kPadY + t + 1;
-                    const bool drow_ok = t + 1 < bh_eff + 2 * kPadY && dn >= 0 && dn < kP;
 #pragma unroll
-                    for (int l = 0; l < LPTD; ++l)
-                        if (d_lds[l] >= 0)
-                            dring[dslot * DROW_UNITS + d_lds[l]] =
-                                (drow_ok && d_ok[l]) ? dpre[(uu + 1) % PF][l] : zero4;
+                    for (int l = 0; l < LPTD; ++l) dring[dslot * DROW_UNITS + d_lds[l]] = dpre[(uu + 1) % PF][l];
                 }
 
                 // 5. multiply: weight gradient ...
@@ -553,11 +600,13 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
 #pragma unroll
                     for (int e = 0; e < 4; ++e) scratch[e * 32 + (lane - 32)] = acc[r + 1][nb][e];
                 }
+                wave_sync();  // lanes 32-63 stored, lanes 0-31 load
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     total[nb][e] = 0.f;
                     if (lane < 32) total[nb][e] = acc[r][nb][e] + scratch[e * 32 + lane];
                 }
+                wave_sync();  // the scratch is free for the next tap pair
             }
             if (TS > 1) {
                 if (ws > 0 && lane < 32) {
@@ -592,15 +641,18 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
         }
         if (wave_active && ws == 0) {
             float* gout = grad_weight + (long long)gglob * GROUP_FLOATS;
+            wave_sync();  // lanes 0-31 staged the sums, all lanes read them
 #pragma unroll
             for (int i = 0; i < kR * kS; ++i) atomic_add_f32(gout + 64 * i + lane, gstage[64 * i + lane]);
         }
 #if SPIO_HAS_BIAS
         {
+            wave_sync();
             if (lane >= 32) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) scratch[e * 32 + (lane - 32)] = accb[e];
             }
+            wave_sync();
             float* bslots = reinterpret_cast<float*>(lds) + WAVES * SCRATCH_FLOATS + RED_FLOATS +
                             GB * GROUP_FLOATS;  // [wave][8]
             if ((lane & 47) == 0) {

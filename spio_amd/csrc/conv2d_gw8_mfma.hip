@@ -459,9 +459,13 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
 
             // 2. multiply source row t into the live output rows.  The fragment reads are issued
             //    first; the previous step's output row is stored while they are in flight.  Rows
-            //    above and below the image are rows of zeros in the ring: no special case.
+            //    above and below the image are rows of zeros in the ring; their products are
+            //    skipped (a scalar branch around LDS reads and MFMAs only: with a 7-row filter on a
+            //    14-row image they would be 6 of 20 steps).
+            const int hcur = p0 + t - EPY;
+            const bool row_live = hcur >= 0 && hcur < SH;
             spio_half8 bfrag[TPW][KB];
-            {
+            if (row_live) {
                 const lds_u4p rrow = ring + rbuf * RING_ROW_UNITS + frag_unit;
 #pragma unroll
                 for (int i = 0; i < TPW; ++i) {
@@ -477,17 +481,19 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
                 }
             }
             if (!kFullUnroll || t >= kR) store_output_row(t - 1, (uu + 1) & 1);
+            if (row_live) {
 #pragma unroll
-            for (int i = 0; i < TPW; ++i) {
-                const int tile = ws + TS * i;
-                if (TS == 1 || tile < WT) {
+                for (int i = 0; i < TPW; ++i) {
+                    const int tile = ws + TS * i;
+                    if (TS == 1 || tile < WT) {
 #pragma unroll
-                    for (int a = 0; a < NACC; ++a) {
-                        const int d = pmod(ph - 2 * a, NS);
+                        for (int a = 0; a < NACC; ++a) {
+                            const int d = pmod(ph - 2 * a, NS);
 #pragma unroll
-                        for (int u = 0; u < KB; ++u)
-                            acc[i][a] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                                wfrag[d][u], bfrag[i][u], acc[i][a], 0, 0, 0);
+                            for (int u = 0; u < KB; ++u)
+                                acc[i][a] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                    wfrag[d][u], bfrag[i][u], acc[i][a], 0, 0, 0);
+                        }
                     }
                 }
             }

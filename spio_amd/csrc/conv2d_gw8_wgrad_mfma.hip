@@ -451,11 +451,13 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
 #pragma unroll
                     for (int e = 0; e < 4; ++e) scratch[e * 32 + (lane - 32)] = acc[r + 1][nb][e];
                 }
+                wave_sync();  // lanes 32-63 stored, lanes 0-31 load
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     total[nb][e] = 0.f;
                     if (lane < 32) total[nb][e] = acc[r][nb][e] + scratch[e * 32 + lane];
                 }
+                wave_sync();  // the scratch is free for the next tap pair
             }
             if (TS > 1) {
                 if (ws > 0 && lane < 32) {
@@ -486,10 +488,12 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
 #pragma unroll
                         for (int e = 0; e < 4; ++e) stage[(nb * 4 + e) * 32 + lane] = total[nb][e];
                 }
+                wave_sync();  // lanes 0-31 staged, all lanes load
                 const spio_float4* stage4 = reinterpret_cast<const spio_float4*>(stage);
                 spio_float4* out4 = reinterpret_cast<spio_float4*>(out) + r * NBLK * 32;
 #pragma unroll
                 for (int i = lane; i < NBLK * 32; i += 64) __builtin_nontemporal_store(stage4[i], out4 + i);
+                wave_sync();  // the scratch is free for the next filter row
             }
 #else
             if (wave_active && ws == 0 && lane < 32) {
@@ -510,9 +514,10 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
         // One wave per group adds the group's R*S*64 sums into grad_weight: every atomic
         // instruction covers 64 consecutive floats (two full 128-byte lines), which the memory
         // system retires several times faster than the scattered half-lines of the accumulator
-        // layout.  The wave reads back what it wrote itself, so no barrier is needed.
+        // layout.  The wave reads back what it wrote itself, so a wave-level sync is enough.
         if (wave_active && ws == 0) {
             float* gout = out + (long long)gglob * GROUP_FLOATS;
+            wave_sync();  // lanes 0-31 staged the sums, all lanes read them
 #pragma unroll
             for (int i = 0; i < kR * kS; ++i) atomic_add_f32(gout + 64 * i + lane, gstage[64 * i + lane]);
         }
@@ -524,10 +529,12 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
         // values with a single atomic instruction: atomics of different workgroups to the same
         // 128-byte line retire one after the other, so their number per line is what counts.
         {
+            wave_sync();
             if (lane >= 32) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) scratch[e * 32 + (lane - 32)] = accb[e];
             }
+            wave_sync();
             float* bslots = reinterpret_cast<float*>(lds) + WAVES * SCRATCH_FLOATS + RED_FLOATS +
                             (SPIO_PARTIALS ? 0 : GB * GROUP_FLOATS);  // [wave][8]
             if ((lane & 47) == 0) {

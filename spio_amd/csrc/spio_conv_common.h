@@ -63,6 +63,16 @@ SPIO_DEVICE void block_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 }
 
+// Orders the LDS accesses of the lanes of one wave: what some lanes stored before it is what
+// other lanes of the same wave load after it.  The hardware executes the LDS operations of a
+// wave in order anyway; this keeps the compiler from moving them across (the store and the load
+// sit under disjoint lane masks, so nothing else tells it they depend on each other).
+SPIO_DEVICE void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // Streaming accesses: activations are touched once per kernel, so they are
 // loaded and stored with the non-temporal hint (measured on MI355X: a plain
 // 16-byte-per-lane copy gains about 10% from it).

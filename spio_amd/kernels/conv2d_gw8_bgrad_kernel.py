@@ -31,6 +31,7 @@ MAX_LDS_BYTES = 128 * 1024
 MAX_LOADS_PER_THREAD = 4
 MAX_REGISTERS = 224  # estimated fragments + accumulators + prefetch buffers, in 32-bit registers
 GEOMETRIES_PER_HEIGHT = 6
+MAX_UNROLLED_STEPS = 40  # SPIO_MAX_UNROLL of the kernel: longer step loops run in chunks
 
 
 @dataclass(frozen=True)
@@ -47,6 +48,10 @@ class Conv2dGw8BgradConfig:
         prefetch: rows of global loads in flight ahead of the computed row (even).
         split: waves per group; they share the 32-pixel chunks (weight gradient) and the
             16-pixel tiles (data gradient) of a row.
+        halo_cached: 1 = rows shared with the neighbouring row blocks are loaded with the default
+            cache policy (the second reader can hit in L2), the others with the non-temporal hint.
+        xcd_chunk: consecutive tiles that go to the same XCD before the next run goes to the next
+            one; 0 = one contiguous range of tiles per XCD.
     """
 
     groups: int = 4
@@ -55,6 +60,8 @@ class Conv2dGw8BgradConfig:
     block_n_iters: int = 1
     prefetch: int = 4
     split: int = 1
+    halo_cached: int = 1
+    xcd_chunk: int = 4
 
 
 def bgrad_is_supported(params: Conv2dGw8Params) -> bool:
@@ -84,7 +91,8 @@ def bgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig) -> Dic
     gsd = fpd + ((9 - fpd % 16) + 16) % 16
     nrd = 4 if (params.has_bias and r == 1) else 2 * ((r + 2) // 2)
     threads = 64 * gb * ts
-    ring_units = 2 * gb * gsx + nrd * (gb * gsd + ((4 - (gb * gsd) % 16) + 16) % 16)
+    # every ring row carries a spare unit behind its last group (see the kernel)
+    ring_units = 2 * (gb * gsx + 1) + nrd * (gb * gsd + 1 + ((4 - (gb * gsd + 1) % 16) + 16) % 16)
     out_row_bytes = 16 * wt * (gb * 16 + 16)
     stream_bytes = ring_units * 16 + 2 * out_row_bytes
     filter_bytes = gb * 8 * r * s * 16
@@ -103,6 +111,7 @@ def bgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig) -> Dic
         NBLK=nblk, KC=kc, CPW=cpw, WT=wt, TPW=tpw, THREADS=threads,
         LDS_BYTES=max(stream_bytes, filter_bytes, publish_bytes),
         LPTX=lptx, LPTD=lptd, REGISTERS=registers,
+        STEPS=bh + 3 * params.padding_h + (1 if params.has_bias and r == 1 else 0),
         BH=bh, GBLKS=divup(params.groups, gb), PBLKS=divup(params.p, bh), NBLKS=divup(params.n, nb * iters),
         PIXEL_EFF=(nb * params.q) / (32.0 * kc),
     )  # fmt: skip
@@ -124,6 +133,11 @@ def _config_is_legal(params, config) -> bool:
         and g["REGISTERS"] <= MAX_REGISTERS
         and config.prefetch >= 2
         and config.prefetch % 2 == 0
+        # The chunked form of the step loop gave wrong grad_input values now and then in
+        # 16-wave workgroups (56-row blocks, lanes 12-15 of the 16-lane groups; cause not found;
+        # 8-wave workgroups and the unrolled form are clean in the same tests): not offered.
+        and (g["STEPS"] <= MAX_UNROLLED_STEPS or g["THREADS"] <= 512)
+        and config.block_n * params.c * params.h * params.w * 2 < 2**31
     )
 
 
@@ -161,8 +175,12 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None) -> List[Conv2dGw8Bgr
                             geometries.append((_score(params, cfg, num_cus), cfg))
         geometries.sort(key=lambda sc: sc[0])
         configs += [cfg for _, cfg in geometries[:GEOMETRIES_PER_HEIGHT]]
-    # a shallower pipeline for the first few: it wins where rows are short
-    configs += [replace(cfg, prefetch=2) for cfg in configs[:GEOMETRIES_PER_HEIGHT]]
+    # a shallower and a deeper pipeline for the first few: the shallow one wins where rows are short
+    first = configs[:GEOMETRIES_PER_HEIGHT]
+    configs += [replace(cfg, prefetch=2) for cfg in first]
+    configs += [replace(cfg, prefetch=8) for cfg in first[:3] if _config_is_legal(params, replace(cfg, prefetch=8))]
+    # ... and the other memory-system policies
+    configs += [replace(cfg, halo_cached=hc, xcd_chunk=ch) for cfg in first[:2] for hc, ch in ((0, 4), (1, 0))]
     return configs
 
 
@@ -174,6 +192,7 @@ def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig, _dev
     defines.update(SPIO_GB=config.groups, SPIO_BH=g["BH"], SPIO_NB=config.block_n,
                    SPIO_ITERS=config.block_n_iters,
                    SPIO_PF=config.prefetch, SPIO_TS=config.split,
+                   SPIO_HALO_CACHED=config.halo_cached, SPIO_XCD_CHUNK=config.xcd_chunk,
                    SPIO_HAS_BIAS=int(params.has_bias))  # fmt: skip
     return KernelSpec(defines, LaunchParams(grid=g["NUM_BLOCKS"], block=g["THREADS"]), SOURCE, notes=g)
 

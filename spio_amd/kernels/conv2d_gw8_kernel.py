@@ -112,8 +112,8 @@ def _mfma_config_is_legal(params, config, igrad) -> bool:
         and g["LPT"] <= MAX_LOADS_PER_THREAD
         and g["TPW"] * g["NACC"] <= MAX_ACCUMULATORS
         and config.prefetch >= 2
-        # longer loops run in chunks of lcm(row slots, prefetch) steps: keep those chunks small
-        and (g["STEPS"] <= MAX_UNROLLED_STEPS or g["UNROLL"] <= 16)
+        # the step loop is always unrolled completely (exact counts of outstanding loads/stores)
+        and g["STEPS"] <= MAX_UNROLLED_STEPS
         # 32-bit buffer offsets inside a workgroup's image block
         and config.block_n * params.c * max(params.h * params.w, params.p * params.q) * 2 < 2**31
         and g["LPT"] * config.prefetch <= 24

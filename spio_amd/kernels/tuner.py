@@ -14,6 +14,16 @@ Environment:
   SPIO_TUNE=1      sweep on a miss (default)
   SPIO_TUNE=force  sweep even when a record exists
   SPIO_TUNE_DB     path of the record file (default: <cache dir>/tune/<arch>_<CUs>cu.json)
+  SPIO_TUNE_MAX_CONFIGS  how many configurations (the first ones of the ranked list) a sweep that
+                   starts inside an operator call may try (default 8); `python -m spio_amd.tune`
+                   and `tune_model` always try all of them
+
+A sweep never starts while the current stream is being captured into a HIP graph (it allocates
+and synchronises): the first configuration is used then, and nothing is recorded.
+
+Before a winner is recorded its output on the synthetic arguments is compared with that of an
+independent implementation (the direct kernel of the family where there is one, else the
+candidate that differs most in tile geometry); a winner that disagrees is discarded.
 """
 
 import dataclasses
@@ -34,6 +44,42 @@ _PACKAGE_RECORDS = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tun
 # the 256 MB memory-side cache.
 ROTATION_BYTES = 600 * 1024 * 1024
 MAX_ROTATION_SETS = 8
+DEFAULT_ON_MISS_CONFIGS = 8
+
+
+def _on_miss_limit() -> int:
+    try:
+        return max(1, int(os.environ.get("SPIO_TUNE_MAX_CONFIGS", DEFAULT_ON_MISS_CONFIGS)))
+    except ValueError:
+        return DEFAULT_ON_MISS_CONFIGS
+
+
+def _stream_is_capturing() -> bool:
+    try:
+        import torch  # pylint: disable=import-outside-toplevel
+
+        return bool(torch.cuda.is_current_stream_capturing())
+    except Exception:  # pylint: disable=broad-except
+        return False
+
+
+def _outputs_agree(a, b) -> bool:
+    """Loose agreement of two kernels' results on the same arguments (fp16 tensors: the
+    operator's tolerance; fp32 sums: relative to the largest value)."""
+    import torch  # pylint: disable=import-outside-toplevel
+
+    for x, y in zip(a, b):
+        if not (torch.isfinite(x).all() and torch.isfinite(y).all()):
+            return False
+        x32, y32 = x.float(), y.float()
+        scale = float(y32.abs().max().clamp_min(1e-6))
+        if x.dtype == torch.float16:
+            ok = torch.allclose(x32, y32, rtol=4e-3, atol=2e-2 * max(1.0, scale / 16.0))
+        else:
+            ok = float((x32 - y32).abs().max()) <= 2e-3 * scale
+        if not ok:
+            return False
+    return True
 
 
 def _mode() -> str:
@@ -133,10 +179,16 @@ class Tuner:
                     return compile_and_load_kernel(
                         kernel_factory, params, config, ordinal, device_attr, **kernel_kwargs
                     )
-            if mode in ("0", "false", "off", "no") or len(configs) == 1:
+            if mode in ("0", "false", "off", "no") or len(configs) == 1 or _stream_is_capturing():
                 return compile_and_load_kernel(
                     kernel_factory, params, configs[0], ordinal, device_attr, **kernel_kwargs
                 )
+            # inside an operator call: only the best-ranked few, so that a model with many new
+            # shapes does not stall (the last entry of a list is its any-shape kernel: keep it as
+            # the independent implementation the winner is checked against)
+            limit = _on_miss_limit()
+            if len(configs) > limit + 1:
+                configs = configs[:limit] + [configs[-1]]
             return self.sweep(kernel_factory, params, ordinal, device_attr, configs, **kernel_kwargs)
 
     def sweep(self, kernel_factory, params, ordinal, device_attr, configs=None, warmup=2,
@@ -159,25 +211,25 @@ class Tuner:
             kernel_factory.make_test_args(params, device, **kernel_kwargs) for _ in range(nsets - 1)
         ]
         results = []
-        best = None
+        timed = []
         for kernel in kernels:
             try:
-                kernel.load(device_ordinal=ordinal)
+                kernel.load(device_ordinal=ordinal, clear_code=False)
                 ms = kernel.time(arg_sets, warmup=warmup, iters=iters)
             except ValueError as e:
                 results.append({"config": config_to_dict(kernel.config), "error": str(e)[:200]})
                 kernel.unload()
                 continue
             results.append({"config": config_to_dict(kernel.config), "us": ms * 1e3})
-            if best is None or ms < best[0]:
-                if best is not None:
-                    best[1].unload()
-                best = (ms, kernel)
-            else:
-                kernel.unload()
-        del arg_sets, first
-        if best is None:
+            timed.append((ms, kernel))
+            kernel.unload()
+        if not timed:
             raise ValueError(f"every configuration of {name} failed: {results}")
+        timed.sort(key=lambda mk: mk[0])
+        best = self._first_valid(kernel_factory, params, timed, first, ordinal, results)
+        del arg_sets, first
+        for _, kernel in timed:
+            kernel.code = None  # loaded or discarded: the code objects are not needed any more
         record = {
             "config": config_to_dict(best[1].config),
             "us": best[0] * 1e3,
@@ -192,6 +244,67 @@ class Tuner:
                 f"({len(configs)} configs, {time.perf_counter() - t0:.1f} s)"
             )
         return best[1]
+
+
+    # -- validation of a sweep's winner ------------------------------------
+    @staticmethod
+    def _run_outputs(kernel_factory, params, kernel, args, ordinal):
+        """Run `kernel` once on copies of the synthetic arguments; returns its output tensors."""
+        import torch  # pylint: disable=import-outside-toplevel
+
+        # outputs come first in every kernel family here: (dst, ...), (dw, ...), (dx, dw, ...);
+        # the gradient kernels of a layer with a bias take grad_bias as their last argument
+        family = kernel.kernel_name.split("__")[0]
+        n_out = 2 if family.endswith("bgrad") else 1
+        trailing_out = family.endswith(("wgrad", "bgrad")) and getattr(params, "has_bias", False)
+        call = list(args)
+        outs = []
+        for i, a in enumerate(call):
+            if not hasattr(a, "numel"):
+                continue
+            if i < n_out or (trailing_out and i == len(call) - 1):
+                call[i] = torch.zeros_like(a)  # accumulated outputs start from zero
+                outs.append(call[i])
+        kernel.load(device_ordinal=ordinal, clear_code=False)
+        try:
+            kernel(*call)
+            torch.cuda.synchronize()
+        finally:
+            kernel.unload()
+        return outs
+
+    def _first_valid(self, kernel_factory, params, timed, args, ordinal, results):
+        """The fastest kernel whose result agrees with an independent implementation; loaded."""
+        if len(timed) == 1:
+            timed[0][1].load(device_ordinal=ordinal, clear_code=False)
+            return timed[0]
+        direct = [k for _, k in timed if getattr(k.config, "variant", "mfma") == "direct"]
+        if direct:
+            reference = direct[0]
+        else:
+            # no any-shape kernel in this family: the candidate furthest from the winner in tile
+            # geometry (most differing configuration fields)
+            w = config_to_dict(timed[0][1].config)
+            reference = max((k for _, k in timed[1:]),
+                            key=lambda k: sum(v != w.get(f) for f, v in config_to_dict(k.config).items()))
+        try:
+            expected = self._run_outputs(kernel_factory, params, reference, args, ordinal)
+        except ValueError:
+            timed[0][1].load(device_ordinal=ordinal, clear_code=False)
+            return timed[0]
+        for ms, kernel in timed:
+            if kernel is reference:
+                kernel.load(device_ordinal=ordinal, clear_code=False)
+                return ms, kernel
+            got = self._run_outputs(kernel_factory, params, kernel, args, ordinal)
+            if _outputs_agree(got, expected):
+                kernel.load(device_ordinal=ordinal, clear_code=False)
+                return ms, kernel
+            results.append({"config": config_to_dict(kernel.config), "rejected": "result differs from "
+                            f"{reference.config}"})  # fmt: skip
+            print(f"spio: sweep of {kernel.kernel_name}: configuration {kernel.config} disagrees with "
+                  f"{reference.config} and was discarded")  # fmt: skip
+        raise ValueError(f"no configuration of {timed[0][1].kernel_name} agrees with {reference.config}")
 
 
 tuner = Tuner()
