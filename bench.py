@@ -1,33 +1,44 @@
 #!/usr/bin/env python3
 """Benchmark of the conv2d_gw8 hot path on one MI355X.
 
-A step is one pass of the hot path over one batch of synthetic input: the
-forward kernel, the data-gradient kernel and the weight-gradient kernel
-(including the zero fill of grad_weight it accumulates into) of one
-convolution shape, launched through the C ABI on torch's current stream with
-every tensor already resident in HBM.  Launches rotate over several buffer
-sets that together exceed the 256 MB memory-side cache, so the rates are HBM
-rates, not cache hits.
+Workloads (--workload):
+  target, cfg1, cfg2, cfg3   one convolution shape.  A step is one pass of the hot path over one
+             batch of synthetic input: the forward kernel, then the backward half as the
+             product's backward op runs it (one fused data+weight gradient kernel where the
+             recorded times say it is faster, else the data-gradient and weight-gradient
+             kernels), including the zero fill of grad_weight.  Everything is launched through
+             the C ABI on torch's current stream with every tensor resident in HBM; launches
+             rotate over buffer sets that together exceed the 256 MB memory-side cache several
+             times, so the rates are HBM rates.
+  cfg4       forward (and backward) at C=64 56x56 3x3 for batch sizes 1..512.
+  cfg5       inference of a ConvNeXt-Tiny-shaped network with gw8 convolutions at batch 128.
 
 The single JSON line printed at the end reports
-  value      effective GB/s of the whole step = algorithmic bytes of the three
-             directions / step time (higher is better); the backward half runs as the
-             product's backward op runs it (fused dgrad+wgrad kernel where that is faster),
-  kernels    per-kernel us, effective GB/s and fraction of the 8 TB/s roofline,
-             timed with HIP events on the launch stream,
-  roofline   the same for the kernel that takes the most time,
-  copy_yardstick  a plain non-temporal copy of the same volume (what HBM gives a read-X/write-X
-             kernel on this device),
+  value      effective GB/s of the whole step = the algorithmic bytes the launched kernels move
+             (a fused backward kernel reads grad_output once and is counted once) / step time;
+             `reference_accounting` prices the same time with the reference's three-direction
+             byte count (scripts/plot_kernel_bench.py:430-435),
+  kernels    per-kernel us (median and min over repeated event-timed blocks), effective GB/s and
+             fraction of the 8 TB/s roofline,
+  roofline   the same for the kernel that takes the most time, with the HBM traffic measured by
+             rocprofv3 counters when a summary for this workload is in profiles/,
+  copy_ceiling  the best of a few tuned streaming copies of the same volume (what HBM gives a
+             read-X/write-X kernel on this device), and the plain copy beside it,
   torch_gpu_conv2d  torch's own grouped conv2d (MIOpen) on the same GPU and shapes,
-  cpu_baseline  the reference's CPU oracle path (torch conv2d fp32, groups=C/8,
-             and its autograd) on the host cores for a bounded sample.
+  cpu_baseline  the reference's CPU oracle path (torch conv2d fp32, groups=C/8, and its
+             autograd) on the host cores for a bounded sample, all threads and one thread.
 
-usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload target|cfg1|cfg2|cfg3]
+The timed region is `--steps` steps between synchronisations, repeated until at least 0.2 s have
+been measured; ms_per_step is the median block, so the sample size does not depend on --steps.
+
+usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 """
 
 import argparse
 import json
 import os
+import re
+import statistics
 import sys
 import time
 
@@ -36,16 +47,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what
-# the same counter reads for the plain copy kernel (profiles/conv2d_gw8_target_hbm_traffic.md).
-MEASURED_TRAFFIC_BYTES = {
-    ("target", "fprop"): 104_710_000,
-    ("target", "dgrad"): 104_720_000,
-    ("target", "wgrad"): 105_510_000,
-    ("target", "bgrad"): 163_270_000,
-}
 CACHE_BYTES = 256 * 1024 * 1024
+MIN_TIMED_SECONDS = 0.2
+METRIC = "conv2d_gw8 effective HBM bandwidth (fwd+dgrad+wgrad step)"
 
 WORKLOADS = {
     # name: (description, params kwargs, weight seed)
@@ -58,6 +62,9 @@ WORKLOADS = {
     "cfg3": ("conv2d_gw8 fwd+dgrad+wgrad N=256 C=256 14x14 7x7 pad3 fp16 NHWC",
              dict(n=256, c=256, h=14, w=14, padding=3, r=7, s=7), 2),
 }  # fmt: skip
+SWEEP_BATCHES = (1, 2, 4, 8, 16, 32, 64, 128, 256, 512)
+NETWORK_WIDTHS = ((96, 56), (192, 28), (384, 14), (768, 7))
+LAUNCH_FLOOR_US = 2.2  # an empty kernel in the same back-to-back loop
 
 
 def parse_args():
@@ -65,11 +72,80 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="target", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="target", choices=sorted(WORKLOADS) + ["cfg4", "cfg5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-torch-gpu-baseline", action="store_true")
-    ap.add_argument("--cpu-sample-batch", type=int, default=8)
+    ap.add_argument("--cpu-sample-batch", type=int, default=32)
     return ap.parse_args()
+
+
+# ------------------------------------------------------------------ helpers
+
+
+def measured_traffic(workload, kernel):
+    """HBM bytes per launch from the rocprofv3 counter summaries in profiles/, or None.
+
+    The summaries carry lines `traffic_bytes <workload> <kernel> <bytes>` (FETCH_SIZE + WRITE_SIZE
+    per dispatch, each scaled by what the same counter reads for the plain copy kernel)."""
+    pdir = os.path.join(ROOT, "profiles")
+    try:
+        names = sorted(os.listdir(pdir))
+    except OSError:
+        return None
+    pat = re.compile(rf"traffic_bytes\s+{re.escape(workload)}\s+{re.escape(kernel)}\s+(\d+)")
+    for name in names:
+        try:
+            with open(os.path.join(pdir, name), "r", encoding="utf-8") as f:
+                m = pat.search(f.read())
+        except OSError:
+            continue
+        if m:
+            return int(m.group(1))
+    return None
+
+
+def rotation_sets(set_bytes):
+    """Buffer sets so that one pass over all of them touches >= 4x the memory-side cache."""
+    return max(2, min(16, -(-4 * CACHE_BYTES // max(set_bytes, 1))))
+
+
+def timed_blocks(run_block, min_seconds=MIN_TIMED_SECONDS, max_blocks=400):
+    """Repeat `run_block()` (which returns the seconds it took) until min_seconds have been
+    measured; returns the list of block times."""
+    times = []
+    total = 0.0
+    while (total < min_seconds or len(times) < 3) and len(times) < max_blocks:
+        t = run_block()
+        times.append(t)
+        total += t
+    return times
+
+
+def time_kernel(kernel, arg_sets, iters):
+    """Median and min microseconds per call over repeated event-timed blocks of `iters` launches."""
+    kernel.time(arg_sets, warmup=10, iters=iters)
+    per_call = []
+    total = 0.0
+    while (total < MIN_TIMED_SECONDS or len(per_call) < 3) and len(per_call) < 400:
+        ms = kernel.time(arg_sets, warmup=0, iters=iters)
+        per_call.append(ms * 1e3)
+        total += ms * 1e-3 * iters
+    return statistics.median(per_call), min(per_call), len(per_call)
+
+
+def kernel_entry(kernel, arg_sets, nbytes, iters):
+    med, mn, blocks = time_kernel(kernel, arg_sets, iters)
+    gbs = nbytes / (med * 1e-6) / 1e9
+    return {
+        "us": round(med, 2),
+        "us_min": round(mn, 2),
+        "blocks": blocks,
+        "bytes": nbytes,
+        "GB/s": round(gbs, 1),
+        "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+        "config": dict(vars(kernel.config)),
+        "kernel": kernel.kernel_name,
+    }
 
 
 def make_buffers(params, seed, nsets, device):
@@ -97,28 +173,62 @@ def make_buffers(params, seed, nsets, device):
     return w, sets
 
 
-def copy_yardstick(nbytes, nsets, device, iters):
-    """Rate of a plain 16-byte-per-lane non-temporal copy of `nbytes` in and `nbytes` out."""
+def copy_ceiling(nbytes, device, iters):
+    """What HBM gives a kernel that reads `nbytes` and writes `nbytes`: the plain one-load-one-store
+    copy and a few tuned grid-stride variants (independent loads in flight per lane, workgroup
+    size, grid as a multiple of the CU count); the best is the ceiling."""
     import torch
 
     from spio_amd.compiler.compile_kernel import compile_and_load_kernel
+    from spio_amd.hip import get_device_attributes
 
-    _module, fn = compile_and_load_kernel("spio_stream_copy", "stream_copy.hip", {}, device.index or 0)
+    cus = get_device_attributes(device.index or 0).multiprocessor_count
     n = nbytes // 16
+    nsets = rotation_sets(2 * nbytes)
     sets = []
     for _ in range(nsets):
         src = torch.randint(0, 2**31 - 1, (n * 4,), dtype=torch.int32, device=device)
-        sets.append((torch.empty_like(src), src, n))
+        sets.append((torch.empty_like(src), src))
     stream = torch.cuda.current_stream(device).cuda_stream
-    ms = fn.launch_timed(((n + 255) // 256, 1, 1), (256, 1, 1), sets, 0, stream, 5, iters)
+
+    def run(fn, grid, threads, args_of):
+        asets = [args_of(d, s) for d, s in sets]
+        fn.launch_timed((grid, 1, 1), (threads, 1, 1), asets, 0, stream, 10, iters)
+        per_call, total = [], 0.0
+        while (total < MIN_TIMED_SECONDS / 2 or len(per_call) < 3) and len(per_call) < 200:
+            ms = fn.launch_timed((grid, 1, 1), (threads, 1, 1), asets, 0, stream, 0, iters)
+            per_call.append(ms * 1e3)
+            total += ms * 1e-3 * iters
+        return statistics.median(per_call)
+
+    variants = []
+    _m0, plain = compile_and_load_kernel("spio_stream_copy", "stream_copy.hip", {}, device.index or 0)
+    us = run(plain, (n + 255) // 256, 256, lambda d, s: (d, s, n))
+    variants.append({"kernel": "spio_stream_copy", "threads": 256, "unroll": 1, "grid": (n + 255) // 256,
+                     "us": round(us, 2), "GB/s": round(2 * n * 16 / us / 1e3, 1)})  # fmt: skip
+    keep = [_m0]
+    for threads, unroll, mult in ((512, 1, 16), (256, 2, 16), (256, 4, 8), (1024, 1, 8), (512, 2, 4), (256, 8, 4)):
+        chunks = n // (threads * unroll)
+        if chunks == 0:
+            continue
+        grid = min(chunks, cus * mult)
+        defines = {"SPIO_COPY_THREADS": threads, "SPIO_COPY_UNROLL": unroll}
+        m, fn = compile_and_load_kernel("spio_stream_copy_strided", "stream_copy.hip", defines, device.index or 0)
+        keep.append(m)
+        us = run(fn, grid, threads, lambda d, s, g=grid: (d, s, n, g))
+        variants.append({"kernel": "spio_stream_copy_strided", "threads": threads, "unroll": unroll,
+                         "grid": grid, "us": round(us, 2), "GB/s": round(2 * n * 16 / us / 1e3, 1)})  # fmt: skip
     del sets
+    best = max(variants, key=lambda v: v["GB/s"])
     return {
-        "kernel": "spio_stream_copy",
-        "us": round(ms * 1e3, 2),
         "bytes": 2 * n * 16,
-        "GB/s": round(2 * n * 16 / (ms * 1e-3) / 1e9, 1),
-        "note": "plain non-temporal copy of one activation tensor in and one out: the HBM rate "
-                "a read-X/write-X kernel reaches on this device",
+        "buffer_sets": nsets,
+        "best": best,
+        "plain": variants[0],
+        "frac_of_hbm_peak": round(best["GB/s"] / HBM_PEAK_GBS, 4),
+        "variants": variants,
+        "note": "non-temporal copies of one activation tensor in and one out over rotating buffers: "
+                "the HBM rate a read-X/write-X kernel reaches on this device",
     }
 
 
@@ -164,8 +274,28 @@ def torch_gpu_conv2d(params, sets, w, iters):
     return out
 
 
+def physical_cores():
+    """Distinct (package, core) pairs in /proc/cpuinfo, or None."""
+    try:
+        seen, phys, core = set(), None, None
+        with open("/proc/cpuinfo", "r", encoding="utf-8") as f:
+            for line in f:
+                if line.startswith("physical id"):
+                    phys = line.split(":")[1].strip()
+                elif line.startswith("core id"):
+                    core = line.split(":")[1].strip()
+                elif not line.strip():
+                    if phys is not None and core is not None:
+                        seen.add((phys, core))
+                    phys = core = None
+        return len(seen) or None
+    except OSError:
+        return None
+
+
 def cpu_baseline(params_kwargs, seed, sample_batch):
-    """The reference's oracle path on the host cores, on a bounded sample of the workload."""
+    """The reference's oracle path on the host cores, on a bounded sample of the workload:
+    all threads (the `value`) and one thread."""
     import torch
 
     from oracle import conv2d_gw8_oracle as oracle
@@ -175,22 +305,29 @@ def cpu_baseline(params_kwargs, seed, sample_batch):
     kw["n"] = min(kw["n"], sample_batch)
     p = Conv2dGw8Params(**kw)
     x, w, _b, dy = oracle.make_args(p.n, p.c, p.h, p.w, p.r, p.s, p.padding_h, p.padding_w, False, seed)
-    threads = torch.get_num_threads()
+    stats = Conv2dStats(p, output_names=["output", "grad_input", "grad_weight"])
 
     def one_pass():
         oracle.fprop_torch(x, w, None, p.padding_h, p.padding_w)
         oracle.grads_torch(x, w, None, dy, p.padding_h, p.padding_w)
 
-    one_pass()
-    times = []
-    t_end = time.perf_counter() + 15.0
-    while len(times) < 5 or (time.perf_counter() < t_end and len(times) < 30):
-        t0 = time.perf_counter()
+    def measure(budget_s, min_runs, max_runs):
         one_pass()
-        times.append(time.perf_counter() - t0)
-    times.sort()
-    med = times[len(times) // 2]
-    stats = Conv2dStats(p, output_names=["output", "grad_input", "grad_weight"])
+        times = []
+        t_end = time.perf_counter() + budget_s
+        while len(times) < min_runs or (time.perf_counter() < t_end and len(times) < max_runs):
+            t0 = time.perf_counter()
+            one_pass()
+            times.append(time.perf_counter() - t0)
+        return statistics.median(times), len(times)
+
+    threads = torch.get_num_threads()
+    med, runs = measure(12.0, 5, 400)
+    torch.set_num_threads(1)
+    try:
+        med1, runs1 = measure(8.0, 3, 100)
+    finally:
+        torch.set_num_threads(threads)
     return {
         "value": round(stats.bytes / med / 1e9, 3),
         "unit": "GB/s",
@@ -199,29 +336,24 @@ def cpu_baseline(params_kwargs, seed, sample_batch):
         "sample": (
             f"torch.nn.functional.conv2d fp32 groups=C/8 forward + autograd grads (the function the "
             f"reference's tests use as oracle), batch {p.n} of {params_kwargs['n']} of the same "
-            f"workload, median of {len(times)} passes, {med * 1e3:.1f} ms/pass, "
-            f"{os.cpu_count()} logical CPUs visible"
+            f"workload, median of {runs} passes, {med * 1e3:.1f} ms/pass on {threads} threads"
         ),
         "ms_per_pass": round(med * 1e3, 3),
+        "single_thread": {"value": round(stats.bytes / med1 / 1e9, 3), "unit": "GB/s", "cores": 1,
+                          "ms_per_pass": round(med1 * 1e3, 3), "passes": runs1},
+        "logical_cpus": os.cpu_count(),
+        "physical_cores": physical_cores(),
     }
 
 
-def main():
-    args = parse_args()
-    if args.gpus != 1:
-        print(
-            "bench.py measures one GPU: the conv2d_gw8 path has no multi-GPU component "
-            f"(--gpus {args.gpus} is not supported; run with --gpus 1).",
-            file=sys.stderr,
-        )
-        sys.exit(2)
+# ------------------------------------------------------------------ workloads
 
+
+def bench_conv(args, device):
+    """One convolution shape: the fwd + backward step, its kernels, the yardsticks."""
     import torch
 
-    if not torch.cuda.is_available():
-        print("bench.py needs a GPU (torch.cuda.is_available() is False).", file=sys.stderr)
-        sys.exit(1)
-
+    from spio_amd.functional import fused_backward_kernel
     from spio_amd.kernels import (
         Conv2dGw8Params,
         Conv2dStats,
@@ -231,25 +363,19 @@ def main():
 
     desc, pkw, seed = WORKLOADS[args.workload]
     params = Conv2dGw8Params(**pkw)
-    device = torch.device("cuda", 0)
-    torch.cuda.set_device(device)
-
-    set_bytes = 2 * (2 * params.n * params.c * params.h * params.w + 2 * params.n * params.c * params.p * params.q)
-    nsets = max(2, min(8, -(-3 * CACHE_BYTES // set_bytes)))
+    act_bytes = 2 * params.n * params.c * params.h * params.w
+    out_bytes = 2 * params.n * params.c * params.p * params.q
+    # the forward kernel alone touches x and y of a set: size the rotation for that
+    nsets = rotation_sets(act_bytes + out_bytes)
     w, sets = make_buffers(params, seed, nsets, device)
 
-    # First use: tunes (or reads the recorded choice), compiles and loads.
+    # First use: reads the recorded choice (or tunes), compiles and loads.
     t0 = time.perf_counter()
     k_fwd = conv2d_gw8_kernel_factory.get_kernel(params, device)
     k_dgrad = conv2d_gw8_kernel_factory.get_kernel(params, device, igrad=True)
     k_wgrad = conv2d_gw8_wgrad_kernel_factory.get_kernel(params, device)
-    setup_s = time.perf_counter() - t0
-
-    # The backward half of the step runs the way the product's backward op runs it: one fused
-    # data+weight gradient kernel where the recorded times say it beats the two separate ones.
-    from spio_amd.functional import fused_backward_kernel
-
     k_fused = fused_backward_kernel(params, device)
+    setup_s = time.perf_counter() - t0
 
     def step(i):
         s = sets[i % nsets]
@@ -264,12 +390,17 @@ def main():
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(i)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed * 1e3 / args.steps
+
+    def block():
+        t = time.perf_counter()
+        for i in range(args.steps):
+            step(i)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t
+
+    blocks = timed_blocks(block)
+    ms_per_step = statistics.median(blocks) * 1e3 / args.steps
+    ms_per_step_min = min(blocks) * 1e3 / args.steps
 
     # The same steps replayed from HIP graphs (one graph per buffer set): what a caller that
     # captures its training step gets; reported beside the eager figure, which stays `value`.
@@ -288,11 +419,15 @@ def main():
         for i in range(args.warmup):
             graphs[i % nsets].replay()
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(args.steps):
-            graphs[i % nsets].replay()
-        torch.cuda.synchronize()
-        graph_ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+        def gblock():
+            t = time.perf_counter()
+            for i in range(args.steps):
+                graphs[i % nsets].replay()
+            torch.cuda.synchronize()
+            return time.perf_counter() - t
+
+        graph_ms_per_step = statistics.median(timed_blocks(gblock)) * 1e3 / args.steps
         del graphs
     except Exception as e:  # pylint: disable=broad-except
         print(f"bench.py: HIP graph replay skipped: {type(e).__name__}: {e}", file=sys.stderr)
@@ -304,57 +439,38 @@ def main():
         "dgrad": Conv2dStats(params, output_names="grad_input"),
         "wgrad": Conv2dStats(params, output_names="grad_weight"),
     }
-    arg_sets = {
-        "fprop": (k_fwd, [(s["y"], s["x"], w, None) for s in sets]),
-        "dgrad": (k_dgrad, [(s["dx"], s["dy"], w, None) for s in sets]),
-        "wgrad": (k_wgrad, [(s["dw"], s["x"], s["dy"]) for s in sets]),
+    nbytes = {
+        "fprop": st["fprop"].bytes,
+        "dgrad": st["dgrad"].bytes,
+        # grad_weight is fp32 on the device
+        "wgrad": st["wgrad"].bytes_read + st["wgrad"].grad_weight_bytes_written_fp32,
     }
-    kernels = {}
-    for name, (kernel, asets) in arg_sets.items():
-        ms = kernel.time(asets, warmup=5, iters=iters)
-        nbytes = st[name].bytes
-        if name == "wgrad":  # grad_weight is fp32 on the device
-            nbytes = st[name].bytes_read + st[name].grad_weight_bytes_written_fp32
-        gbs = nbytes / (ms * 1e-3) / 1e9
-        kernels[name] = {
-            "us": round(ms * 1e3, 2),
-            "bytes": nbytes,
-            "GB/s": round(gbs, 1),
-            "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
-            "config": {k: v for k, v in vars(kernel.config).items()},
-            "kernel": kernel.kernel_name,
-        }
-    # `value` keeps the reference's accounting (the algorithmic bytes of the three directions,
-    # scripts/plot_kernel_bench.py:430-435) whether or not the backward half is fused, so it is a
-    # pure time metric; the fused kernel's own roofline entry counts grad_output once.
-    step_bytes = sum(k["bytes"] for k in kernels.values())
-    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    nbytes["bgrad"] = nbytes["dgrad"] + nbytes["wgrad"] - out_bytes  # grad_output is read once
+    kernels = {
+        "fprop": kernel_entry(k_fwd, [(s["y"], s["x"], w, None) for s in sets], nbytes["fprop"], iters),
+        "dgrad": kernel_entry(k_dgrad, [(s["dx"], s["dy"], w, None) for s in sets], nbytes["dgrad"], iters),
+        "wgrad": kernel_entry(k_wgrad, [(s["dw"], s["x"], s["dy"]) for s in sets], nbytes["wgrad"], iters),
+    }
     if k_fused is not None:
-        ms = k_fused.time([(s["dx"], s["dw"], s["x"], s["dy"], w) for s in sets], warmup=5, iters=iters)
-        nbytes = (st["dgrad"].bytes + st["wgrad"].bytes_read + st["wgrad"].grad_weight_bytes_written_fp32
-                  - 2 * params.n * params.c * params.p * params.q)  # grad_output is read once
-        gbs = nbytes / (ms * 1e-3) / 1e9
-        kernels["bgrad"] = {
-            "us": round(ms * 1e3, 2),
-            "bytes": nbytes,
-            "GB/s": round(gbs, 1),
-            "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
-            "config": {k: v for k, v in vars(k_fused.config).items()},
-            "kernel": k_fused.kernel_name,
-            "note": "fused dgrad+wgrad as the backward op runs it for this shape; replaces the "
-                    "dgrad and wgrad launches in the timed step",
-            # the same time priced with the bytes the two separate kernels need for this work
-            "unfused_accounting": {
-                "bytes": kernels["dgrad"]["bytes"] + kernels["wgrad"]["bytes"],
-                "GB/s": round((kernels["dgrad"]["bytes"] + kernels["wgrad"]["bytes"]) / (ms * 1e-3) / 1e9, 1),
-                "frac_of_hbm_peak": round(
-                    (kernels["dgrad"]["bytes"] + kernels["wgrad"]["bytes"]) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4
-                ),
-            },
+        kernels["bgrad"] = kernel_entry(
+            k_fused, [(s["dx"], s["dw"], s["x"], s["dy"], w) for s in sets], nbytes["bgrad"], iters
+        )
+        kernels["bgrad"]["note"] = ("fused dgrad+wgrad as the backward op runs it for this shape; replaces "
+                                    "the dgrad and wgrad launches in the timed step")
+        ref_bytes = nbytes["dgrad"] + nbytes["wgrad"]
+        kernels["bgrad"]["reference_accounting"] = {
+            "bytes": ref_bytes,
+            "GB/s": round(ref_bytes / (kernels["bgrad"]["us"] * 1e-6) / 1e9, 1),
+            "note": "the same time priced with the bytes the two separate kernels need for this work",
         }
 
-    in_step = [n for n in kernels if (n in ("fprop", "bgrad") if k_fused is not None else n != "bgrad")]
+    in_step = ["fprop", "bgrad"] if k_fused is not None else ["fprop", "dgrad", "wgrad"]
+    step_bytes = sum(nbytes[n] for n in in_step)  # what the timed step moves
+    ref_step_bytes = nbytes["fprop"] + nbytes["dgrad"] + nbytes["wgrad"]
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
     dominant = max(in_step, key=lambda n: kernels[n]["us"])
+    for name in kernels:
+        kernels[name]["traffic"] = measured_traffic(args.workload, name)
     roofline = {
         "bound": "hbm",
         "kernel": kernels[dominant]["kernel"],
@@ -362,11 +478,11 @@ def main():
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": kernels[dominant]["frac_of_hbm_peak"],
-        "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, dominant)),
+        "traffic": kernels[dominant]["traffic"],
     }
 
     result = {
-        "metric": "conv2d_gw8 effective HBM bandwidth (fwd+dgrad+wgrad step)",
+        "metric": METRIC,
         "value": round(value, 1),
         "unit": "GB/s",
         "n_gpus": 1,
@@ -383,12 +499,21 @@ def main():
             "params": params.encode(),
             "buffer_sets": nsets,
             "first_use_seconds": round(setup_s, 2),
+            "step_kernels": in_step,
         },
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
-        "value_note": "algorithmic bytes of fprop + dgrad + wgrad (the reference's per-direction accounting) "
-                      "divided by the time of one step as the operators run it"
-                      + ("; the backward half of this step is one fused kernel that reads grad_output once, "
-                         "so the step moves fewer bytes than the numerator counts" if k_fused is not None else ""),
+        "value_note": "algorithmic bytes of the kernels the step launches (" + " + ".join(in_step)
+                      + ") divided by the median time of one step",
+        "timed_blocks": len(blocks),
+        "ms_per_step_min": round(ms_per_step_min, 5),
+        "step_bytes": step_bytes,
+        "reference_accounting": {
+            "bytes": ref_step_bytes,
+            "GB/s": round(ref_step_bytes / (ms_per_step * 1e-3) / 1e9, 1),
+            "note": "the same step time priced with the algorithmic bytes of fprop + dgrad + wgrad as "
+                    "three separate kernels (the reference's per-direction accounting)",
+        },
+        "fprop_frac_of_hbm_peak": kernels["fprop"]["frac_of_hbm_peak"],
         "hip_graph_replay": None if graph_ms_per_step is None else {
             "ms_per_step": round(graph_ms_per_step, 5),
             "value": round(step_bytes / (graph_ms_per_step * 1e-3) / 1e9, 1),
@@ -399,18 +524,225 @@ def main():
     }
     if not args.no_torch_gpu_baseline:
         result["torch_gpu_conv2d"] = torch_gpu_conv2d(params, sets, w, min(iters, 50))
-    del arg_sets
     del sets
     torch.cuda.empty_cache()
-    result["copy_yardstick"] = copy_yardstick(
-        2 * params.n * params.c * params.h * params.w, nsets, device, iters
-    )
-    result["roofline"]["frac_of_copy_rate"] = round(
-        kernels[dominant]["GB/s"] / result["copy_yardstick"]["GB/s"], 4
-    )
+    result["copy_ceiling"] = copy_ceiling(act_bytes, device, iters)
+    best = result["copy_ceiling"]["best"]["GB/s"]
+    result["roofline"]["frac_of_copy_ceiling"] = round(kernels[dominant]["GB/s"] / best, 4)
+    result["fprop_frac_of_copy_ceiling"] = round(kernels["fprop"]["GB/s"] / best, 4)
     if not args.no_cpu_baseline:
         torch.cuda.empty_cache()
         result["cpu_baseline"] = cpu_baseline(pkw, seed, args.cpu_sample_batch)
+    return result
+
+
+def bench_batch_sweep(args, device):
+    """cfg4: the forward kernel (and the backward half) at C=64 56x56 3x3 for N = 1 .. 512: the
+    reference's headline plot, effective bandwidth versus batch size
+    (scripts/profile_blocks.bash:4-5, scripts/plot_kernel_bench.py:417-435)."""
+    import torch
+
+    from spio_amd.functional import fused_backward_kernel
+    from spio_amd.kernels import (
+        Conv2dGw8Params,
+        Conv2dStats,
+        conv2d_gw8_kernel_factory,
+        conv2d_gw8_wgrad_kernel_factory,
+    )
+
+    sweep = []
+    for n in SWEEP_BATCHES:
+        params = Conv2dGw8Params(n=n, c=64, h=56, w=56, padding=1, r=3, s=3)
+        act = 2 * n * 64 * 56 * 56
+        nsets = rotation_sets(2 * act)
+        w, sets = make_buffers(params, 0, nsets, device)
+        iters = 200 if n <= 64 else 60
+        k_fwd = conv2d_gw8_kernel_factory.get_kernel(params, device)
+        fb = Conv2dStats(params, output_names="output").bytes
+        e = kernel_entry(k_fwd, [(s["y"], s["x"], w, None) for s in sets], fb, iters)
+        point = {"N": n, "fprop_us": e["us"], "fprop_GB/s": e["GB/s"], "fprop_frac": e["frac_of_hbm_peak"],
+                 "fprop_bytes": fb, "launch_floor_dominated": e["us"] < 3 * LAUNCH_FLOOR_US}  # fmt: skip
+        k_fused = fused_backward_kernel(params, device)
+        st_w = Conv2dStats(params, output_names="grad_weight")
+        wb = st_w.bytes_read + st_w.grad_weight_bytes_written_fp32
+        db = Conv2dStats(params, output_names="grad_input").bytes
+        if k_fused is not None:
+            bb = db + wb - act
+            b = kernel_entry(k_fused, [(s["dx"], s["dw"], s["x"], s["dy"], w) for s in sets], bb, iters)
+            point.update({"backward": "fused", "backward_us": b["us"], "backward_GB/s": b["GB/s"],
+                          "backward_frac": b["frac_of_hbm_peak"], "backward_bytes": bb})  # fmt: skip
+        else:
+            k_d = conv2d_gw8_kernel_factory.get_kernel(params, device, igrad=True)
+            k_w = conv2d_gw8_wgrad_kernel_factory.get_kernel(params, device)
+            d = kernel_entry(k_d, [(s["dx"], s["dy"], w, None) for s in sets], db, iters)
+            ww = kernel_entry(k_w, [(s["dw"], s["x"], s["dy"]) for s in sets], wb, iters)
+            us = d["us"] + ww["us"]
+            point.update({"backward": "dgrad+wgrad", "backward_us": round(us, 2),
+                          "backward_GB/s": round((db + wb) / us / 1e3, 1),
+                          "backward_frac": round((db + wb) / us / 1e3 / HBM_PEAK_GBS, 4),
+                          "backward_bytes": db + wb})  # fmt: skip
+        sweep.append(point)
+        del sets
+        torch.cuda.empty_cache()
+    at128 = next(p for p in sweep if p["N"] == 128)
+    best = max(sweep, key=lambda p: p["fprop_GB/s"])
+    return {
+        "metric": METRIC,
+        "value": at128["fprop_GB/s"],
+        "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(at128["fprop_us"] * 1e-3, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp16 (fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": "cfg4: conv2d_gw8 forward (and backward) C=64 56x56 3x3 pad1 fp16 NHWC, "
+                               "N in {1..512}; value is the forward kernel at N=128"},
+        "frac_of_hbm_peak": at128["fprop_frac"],
+        "sweep": sweep,
+        "roofline": {"bound": "hbm", "kernel": f"spio_conv2d_gw8_fprop at N={best['N']}",
+                     "achieved": best["fprop_GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": best["fprop_frac"], "traffic": None},
+        "note": f"launch_floor_dominated marks points under {3 * LAUNCH_FLOOR_US:.1f} us: an empty kernel "
+                f"takes {LAUNCH_FLOOR_US} us in the same back-to-back loop",
+    }  # fmt: skip
+
+
+def bench_network(args, device):
+    """cfg5: inference of the ConvNeXt-Tiny-shaped gw8 network at batch 128 (fp16 autocast, channels_last),
+    with the time of its four distinct gw8 convolution shapes and of the channel LayerNorm."""
+    import torch
+
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from convnext_gw8 import ConvNeXtGw8  # pylint: disable=import-error,import-outside-toplevel
+
+    from spio_amd.kernels import Conv2dGw8Params, Conv2dStats, conv2d_gw8_kernel_factory
+    from spio_amd.layers import Conv2dGw8, LayerNorm2d
+    from spio_amd.kernels.layernorm_2d_kernel import LayerNorm2dParams, layernorm_2d_kernel_factory
+
+    batch = 128
+    torch.manual_seed(3)
+    model = ConvNeXtGw8(make_conv=lambda dim: Conv2dGw8(dim, dim, 3, padding=1, groups=dim // 8),
+                        norm2d=LayerNorm2d)  # fmt: skip
+    model = model.to(device).to(memory_format=torch.channels_last).eval()  # fp32 parameters, fp16 autocast
+    gen = torch.Generator().manual_seed(3)
+    images = [torch.randn(batch, 3, 224, 224, generator=gen).half().to(device)
+              .contiguous(memory_format=torch.channels_last) for _ in range(2)]  # fmt: skip
+    with torch.no_grad(), torch.autocast(device_type="cuda", dtype=torch.float16):
+        t0 = time.perf_counter()
+        model(images[0])
+        torch.cuda.synchronize()
+        first_s = time.perf_counter() - t0
+        for i in range(3):
+            model(images[i % 2])
+        torch.cuda.synchronize()
+        iters = max(5, min(args.steps, 20))
+
+        def block():
+            t = time.perf_counter()
+            for i in range(iters):
+                model(images[i % 2])
+            torch.cuda.synchronize()
+            return time.perf_counter() - t
+
+        blocks = timed_blocks(block, min_seconds=1.0, max_blocks=20)
+    ms_iter = statistics.median(blocks) * 1e3 / iters
+
+    convs, total_bytes, total_us = [], 0, 0.0
+    depth = {96: 3, 192: 3, 384: 9, 768: 3}
+    for c, hw in NETWORK_WIDTHS:
+        params = Conv2dGw8Params(n=batch, c=c, h=hw, w=hw, padding=1, r=3, s=3, has_bias=True)
+        nb = Conv2dStats(params, output_names="output").bytes
+        nsets = rotation_sets(nb)
+        k = conv2d_gw8_kernel_factory.get_kernel(params, device)
+        asets = [conv2d_gw8_kernel_factory.make_test_args(params, device) for _ in range(nsets)]
+        e = kernel_entry(k, asets, nb, 100)
+        convs.append({"shape": params.encode(), "count": depth[c], "us": e["us"], "GB/s": e["GB/s"],
+                      "frac_of_hbm_peak": e["frac_of_hbm_peak"], "bytes": nb})  # fmt: skip
+        total_bytes += depth[c] * nb
+        total_us += depth[c] * e["us"]
+        del asets
+        torch.cuda.empty_cache()
+    norms = []
+    for c, hw in NETWORK_WIDTHS:
+        p = LayerNorm2dParams(n=batch, c=c, h=hw, w=hw)
+        k = layernorm_2d_kernel_factory.get_kernel(p, device)
+        nb = 4 * batch * c * hw * hw + 8 * c
+        nsets = rotation_sets(nb)
+        asets = [layernorm_2d_kernel_factory.make_test_args(p, device) for _ in range(nsets)]
+        e = kernel_entry(k, asets, nb, 100)
+        norms.append({"shape": p.encode(), "us": e["us"], "GB/s": e["GB/s"],
+                      "frac_of_hbm_peak": e["frac_of_hbm_peak"], "bytes": nb})  # fmt: skip
+        del asets
+        torch.cuda.empty_cache()
+    value = total_bytes / (total_us * 1e-6) / 1e9
+    slowest = min(convs, key=lambda cv: cv["frac_of_hbm_peak"])
+    result = {
+        "metric": METRIC,
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_iter, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp16 (fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": "cfg5: ConvNeXt-Tiny-shaped network, 3x3 gw8 convolutions, batch 128, 224x224 "
+                               "inference; value is the 18 gw8 convolutions' bytes over their kernel time",
+                   "first_use_seconds": round(first_s, 2)},
+        "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+        "network_ms_per_iter": round(ms_iter, 3),
+        "images_per_second": round(batch / (ms_iter * 1e-3), 1),
+        "gw8_conv_ms_per_iter": round(total_us * 1e-3, 3),
+        "convs": convs,
+        "layernorm_2d": norms,
+        "roofline": {"bound": "hbm", "kernel": "spio_conv2d_gw8_fprop__" + slowest["shape"],
+                     "achieved": slowest["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": slowest["frac_of_hbm_peak"], "traffic": None},
+    }  # fmt: skip
+    if not args.no_cpu_baseline:
+        sample = 2
+        torch.manual_seed(3)
+        cpu_model = ConvNeXtGw8().float().eval()
+        xs = torch.randn(sample, 3, 224, 224, generator=torch.Generator().manual_seed(3))
+        with torch.no_grad():
+            cpu_model(xs)
+            times = []
+            t_end = time.perf_counter() + 15.0
+            while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 20):
+                t0 = time.perf_counter()
+                cpu_model(xs)
+                times.append(time.perf_counter() - t0)
+        med = statistics.median(times)
+        result["cpu_baseline"] = {
+            "value": round(sample / med, 2), "unit": "images/s", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"the same network with nn.Conv2d(groups=C/8) in fp32 on the host, batch {sample} of "
+                      f"{batch}, median of {len(times)} passes, {med * 1e3:.0f} ms/pass",
+            "logical_cpus": os.cpu_count(), "physical_cores": physical_cores(),
+        }  # fmt: skip
+    return result
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(
+            "bench.py measures one GPU: the conv2d_gw8 path has no multi-GPU component "
+            f"(--gpus {args.gpus} is not supported; run with --gpus 1).",
+            file=sys.stderr,
+        )
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (torch.cuda.is_available() is False).", file=sys.stderr)
+        sys.exit(1)
+    device = torch.device("cuda", 0)
+    torch.cuda.set_device(device)
+    if args.workload == "cfg4":
+        result = bench_batch_sweep(args, device)
+    elif args.workload == "cfg5":
+        result = bench_network(args, device)
+    else:
+        result = bench_conv(args, device)
     print(json.dumps(result))
 
 

@@ -1,0 +1,129 @@
+"""LayerNorm over the channels of an NHWC fp16 tensor: parameters, configurations, factory.
+
+The reference ships the device source of such a kernel (spio/src/layernorm_2d.cu:81-222: NHWC
+fp16 in and out, fp32 mean and variance over C per pixel, optional fp32 weight and bias) without
+a Python side; this module gives the re-designed kernel (csrc/layernorm_2d.hip) the same
+factory / cache / tuner plumbing as the convolution kernels.
+
+Kernel arguments: (output, input, weight or None, bias or None).
+"""
+
+import re
+from dataclasses import dataclass
+from typing import List
+
+import torch
+
+from ..util.math import divup
+from .kernel import KernelSpec
+from .kernel_factory import KernelFactory
+from .launch_params import LaunchParams
+
+SOURCE = "layernorm_2d.hip"
+
+
+@dataclass(frozen=True)
+class LayerNorm2dParams:
+    """Shape of one channel LayerNorm: input [n, c, h, w] with channels_last strides."""
+
+    n: int
+    c: int
+    h: int
+    w: int
+    eps: float = 1e-6
+    has_weight: bool = True
+    has_bias: bool = True
+
+    def encode(self) -> str:
+        flags = ("w" if self.has_weight else "nw") + ("b" if self.has_bias else "nb")
+        return f"{self.n}n_{self.c}c_{self.h}h_{self.w}w_{self.eps:g}eps_{flags}".replace("-", "m")
+
+    _PATTERN = re.compile(r"(\d+)n_(\d+)c_(\d+)h_(\d+)w_([0-9.em+]+)eps_(w|nw)(b|nb)$")
+
+    @classmethod
+    def decode(cls, string: str) -> "LayerNorm2dParams":
+        m = cls._PATTERN.match(string)
+        if m is None:
+            raise ValueError("Invalid string representation.")
+        n, c, h, w = (int(v) for v in m.groups()[:4])
+        return cls(n=n, c=c, h=h, w=w, eps=float(m.group(5).replace("m", "-")),
+                   has_weight=m.group(6) == "w", has_bias=m.group(7) == "b")  # fmt: skip
+
+    def validate(self):
+        assert self.n > 0 and self.h > 0 and self.w > 0
+        assert self.c > 0 and self.c % 8 == 0, "channels must be a multiple of 8 (16-byte units)"
+        assert self.c <= 8 * 64 * 4, "at most 2048 channels"
+        assert self.eps > 0
+
+    @property
+    def pixels(self) -> int:
+        return self.n * self.h * self.w
+
+    @property
+    def shape(self):
+        return (self.n, self.c, self.h, self.w)
+
+
+@dataclass(frozen=True)
+class LayerNorm2dConfig:
+    """threads per workgroup, pixel groups in flight per lane, workgroups per compute unit."""
+
+    threads: int = 256
+    unroll: int = 4
+    groups_per_cu: int = 8
+
+
+def lanes_per_pixel(c: int) -> int:
+    units = c // 8
+    lpp = 1
+    while lpp < units and lpp < 64:
+        lpp *= 2
+    return lpp
+
+
+def _get_configs(params: LayerNorm2dParams, _device_attr=None) -> List[LayerNorm2dConfig]:
+    upl = divup(params.c // 8, lanes_per_pixel(params.c))
+    out = []
+    for threads in (256, 512):
+        for unroll in (4, 2, 8):
+            if unroll * upl > 8:
+                continue
+            for per_cu in (8, 4, 16):
+                out.append(LayerNorm2dConfig(threads, unroll, per_cu))
+    return out or [LayerNorm2dConfig(256, 1, 8)]
+
+
+def _get_kernel_spec(params: LayerNorm2dParams, config: LayerNorm2dConfig, device_attr=None) -> KernelSpec:
+    params.validate()
+    cus = getattr(device_attr, "multiprocessor_count", 256) or 256
+    lpp = lanes_per_pixel(params.c)
+    pass_pixels = (64 // lpp) * (config.threads // 64) * config.unroll
+    grid = max(1, min(divup(params.pixels, pass_pixels), cus * config.groups_per_cu))
+    defines = {
+        "SPIO_LN_C": params.c, "SPIO_LN_PIXELS": params.pixels, "SPIO_LN_LPP": lpp,
+        "SPIO_LN_THREADS": config.threads, "SPIO_LN_UNROLL": config.unroll,
+        "SPIO_LN_HAS_WEIGHT": int(params.has_weight), "SPIO_LN_HAS_BIAS": int(params.has_bias),
+        "SPIO_LN_EPS": f"{params.eps:.9g}f", "SPIO_LN_GRID": grid,
+    }  # fmt: skip
+    return KernelSpec(defines, LaunchParams(grid=grid, block=config.threads), SOURCE,
+                      notes={"LPP": lpp, "PASS_PIXELS": pass_pixels})  # fmt: skip
+
+
+def _make_test_args(params: LayerNorm2dParams, device):
+    cl = torch.channels_last
+    x = torch.randn(params.shape, device=device, dtype=torch.float16).contiguous(memory_format=cl)
+    y = torch.empty_like(x)
+    w = torch.randn(params.c, device=device, dtype=torch.float32) if params.has_weight else None
+    b = torch.randn(params.c, device=device, dtype=torch.float32) if params.has_bias else None
+    return (y, x, w, b)
+
+
+layernorm_2d_kernel_factory = KernelFactory(
+    LayerNorm2dParams,
+    LayerNorm2dConfig,
+    None,
+    kernel_name="spio_layernorm_2d",
+    configs=_get_configs,
+    kernel_spec=_get_kernel_spec,
+    make_test_args=_make_test_args,
+)

@@ -36,12 +36,13 @@ def plain_conv(dim):
 
 
 class ConvNeXtGw8(nn.Module):
-    def __init__(self, make_conv=plain_conv, widths=(96, 192, 384, 768), depths=(3, 3, 9, 3), classes=1000):
+    def __init__(self, make_conv=plain_conv, widths=(96, 192, 384, 768), depths=(3, 3, 9, 3), classes=1000,
+                 norm2d=LayerNorm2d):
         super().__init__()
-        layers = [nn.Conv2d(3, widths[0], 4, stride=4), LayerNorm2d(widths[0])]
+        layers = [nn.Conv2d(3, widths[0], 4, stride=4), norm2d(widths[0])]
         for i, (w, d) in enumerate(zip(widths, depths)):
             if i > 0:
-                layers += [LayerNorm2d(widths[i - 1]), nn.Conv2d(widths[i - 1], w, 2, stride=2)]
+                layers += [norm2d(widths[i - 1]), nn.Conv2d(widths[i - 1], w, 2, stride=2)]
             layers += [Block(w, make_conv) for _ in range(d)]
         self.features = nn.Sequential(*layers)
         self.norm = nn.LayerNorm(widths[-1])

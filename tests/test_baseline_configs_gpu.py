@@ -96,13 +96,44 @@ def test_forward_is_linear_in_the_input_at_full_size():
     assert float((lhs - rhs).abs().mean()) < 2e-3
 
 
-def test_batch_sweep_shapes_small_batches():
-    """Forward at C=64, 56x56 for the small-batch end of the sweep (N = 1 .. 16)."""
-    for n in (1, 2, 4, 8, 16):
-        params = Conv2dGw8Params(n=n, c=64, h=56, w=56, padding=1)
-        x, w, _b, _dy = oracle.make_args(n, 64, 56, 56, 3, 3, 1, 1, False, 0, weight_init="kaiming")
-        y = conv2d_gw8(to_gpu(x), to_gpu(w), None, 1, 1, 1, 1, 8)
-        oracle.check_close(y, oracle.fprop_torch(x, w, None, 1, 1), acc_depth=72, what=params.encode())
+@pytest.mark.parametrize("n", [1, 2, 4, 8, 16, 32, 64, 128, 256, 512])
+def test_batch_sweep_forward(n):
+    """Forward at C=64, 56x56 for every batch size of the sweep configuration."""
+    params = Conv2dGw8Params(n=n, c=64, h=56, w=56, padding=1)
+    x, w, _b, _dy = oracle.make_args(n, 64, 56, 56, 3, 3, 1, 1, False, 0, weight_init="kaiming")
+    y = conv2d_gw8(to_gpu(x), to_gpu(w), None, 1, 1, 1, 1, 8)
+    expected = oracle.fprop_torch(x, w, None, 1, 1)
+    oracle.check_close(y, expected, acc_depth=72, what=params.encode())
+    oracle.check_close(y, expected, what=params.encode() + " (north-star tolerance)")
+
+
+@pytest.mark.parametrize("n", [64, 256])
+def test_batch_sweep_backward(n):
+    """Backward at the sweep batch sizes that no other configuration covers."""
+    params = Conv2dGw8Params(n=n, c=64, h=56, w=56, padding=1)
+    x, w, dy, _y, dx, dw = _run(params, 0)
+    depth = Conv2dStats(params, output_names=["grad_input", "grad_weight"]).accumulation_depths
+    dx_e, dw_e, _ = oracle.grads_torch(x, w, None, dy, 1, 1)
+    oracle.check_close(dx, dx_e, acc_depth=depth[0], what=f"N={n} dgrad")
+    oracle.check_close(dw, dw_e, acc_depth=depth[1], what=f"N={n} wgrad")
+
+
+@pytest.mark.parametrize("c,hw", [(96, 56), (192, 28), (384, 14), (768, 7)])
+def test_network_conv_shapes_at_full_batch_with_bias(c, hw):
+    """The four gw8 convolution shapes of the network configuration at batch 128, with bias,
+    forward and backward through the operators with the recorded configurations."""
+    params = Conv2dGw8Params(n=128, c=c, h=hw, w=hw, padding=1, has_bias=True)
+    x, w, b, dy = oracle.make_args(128, c, hw, hw, 3, 3, 1, 1, True, 3, weight_init="kaiming")
+    xg, wg, bg, dyg = to_gpu(x), to_gpu(w), to_gpu(b), to_gpu(dy)
+    y = conv2d_gw8(xg, wg, bg, stride=1, padding_y=1, padding_x=1, groups=c // 8)
+    dx, dw, db = torch.ops.spio.conv2d_gw8_backward(xg, wg, bg, dyg, 1, 1, True, True, True)
+    torch.cuda.synchronize()
+    depth = Conv2dStats(params, output_names=["output", "grad_input", "grad_weight", "grad_bias"]).accumulation_depths
+    oracle.check_close(y, oracle.fprop_torch(x, w, b, 1, 1), acc_depth=depth[0], what=f"{params.encode()} fprop")
+    dx_e, dw_e, db_e = oracle.grads_torch(x, w, b, dy, 1, 1)
+    oracle.check_close(dx, dx_e, acc_depth=depth[1], what=f"{params.encode()} dgrad")
+    oracle.check_close(dw, dw_e, acc_depth=depth[2], what=f"{params.encode()} wgrad")
+    oracle.check_close(db, db_e, acc_depth=depth[3], what=f"{params.encode()} grad_bias")
 
 
 def test_convnext_shaped_network_logits():
@@ -133,3 +164,23 @@ def test_convnext_shaped_network_logits():
             moved = gpu_model(images.cuda().contiguous(memory_format=torch.channels_last)).float().cpu()
         first.weight.copy_(saved)
     assert float((moved - want).abs().max()) > 10 * float((got - want).abs().max())
+
+
+def test_convnext_shaped_network_with_layernorm_kernels():
+    """The same network built directly from Conv2dGw8 and the LayerNorm2d kernel layer, under fp16
+    autocast as the benchmark runs it, against the fp32 CPU model."""
+    from spio_amd.layers import LayerNorm2d
+
+    torch.manual_seed(3)
+    cpu_model = ConvNeXtGw8().eval()
+    images = torch.randn(4, 3, 224, 224).half().float()
+    with torch.no_grad():
+        want = cpu_model(images)
+    gpu_model = ConvNeXtGw8(make_conv=lambda d: Conv2dGw8(d, d, 3, padding=1, groups=d // 8), norm2d=LayerNorm2d)
+    gpu_model.load_state_dict(cpu_model.state_dict())
+    gpu_model = gpu_model.eval().cuda().to(memory_format=torch.channels_last)
+    with torch.no_grad(), torch.autocast(device_type="cuda", dtype=torch.float16):
+        got = gpu_model(images.cuda().contiguous(memory_format=torch.channels_last))
+    got = got.float().cpu()
+    assert float((got - want).abs().max()) < 0.08 * max(1.0, float(want.abs().max()))
+    assert torch.equal(got.argmax(dim=1), want.argmax(dim=1))

@@ -1,0 +1,85 @@
+"""LayerNorm2d kernel (`spio::layernorm_2d`) against torch's layer_norm in fp32 on the CPU.
+
+Contract of the reference's device source spio/src/layernorm_2d.cu:81-222 (NHWC fp16, fp32
+statistics over C per pixel); the reference has no test for it, so torch is the oracle.
+Tolerance: one fp16 rounding of an O(1..10) value plus fp32 statistics: rtol 2e-3, atol 4e-3.
+"""
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from spio_amd.functional import layernorm_2d
+from spio_amd.hip import get_device_attributes
+from spio_amd.kernels import LayerNorm2dParams, layernorm_2d_kernel_factory
+from spio_amd.layers import LayerNorm2d
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [
+    # the four widths of the network benchmark (small batch), then shapes that exercise lanes
+    # without a unit (c/8 not a power of two), two units per lane, and a ragged last pass
+    (4, 96, 56, 56), (4, 192, 28, 28), (8, 384, 14, 14), (16, 768, 7, 7),
+    (3, 8, 5, 7), (2, 40, 9, 9), (1, 1000, 3, 5), (5, 64, 1, 1), (2, 2048, 2, 3),
+]  # fmt: skip
+
+
+def _reference(x, w, b, eps):
+    y = F.layer_norm(x.float().permute(0, 2, 3, 1), (x.shape[1],), w, b, eps)
+    return y.permute(0, 3, 1, 2)
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("affine", ["wb", "w", "none"])
+def test_layernorm_2d_matches_torch(shape, affine):
+    g = torch.Generator().manual_seed(sum(shape))
+    x = (torch.randn(shape, generator=g) * 2 + 0.5).half()
+    c = shape[1]
+    w = torch.randn(c, generator=g) if affine != "none" else None
+    b = torch.randn(c, generator=g) if affine == "wb" else None
+    expected = _reference(x, w, b, 1e-6)
+    xg = x.cuda().contiguous(memory_format=torch.channels_last)
+    out = layernorm_2d(xg, None if w is None else w.cuda(), None if b is None else b.cuda(), 1e-6)
+    assert out.dtype == torch.float16 and out.is_contiguous(memory_format=torch.channels_last)
+    torch.testing.assert_close(out.float().cpu(), expected, rtol=2e-3, atol=4e-3)
+
+
+def test_every_configuration_of_one_shape():
+    attr = get_device_attributes(0)
+    params = LayerNorm2dParams(n=3, c=192, h=13, w=11)
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(params.shape, generator=g).half()
+    w, b = torch.randn(192, generator=g), torch.randn(192, generator=g)
+    expected = _reference(x, w, b, params.eps)
+    xg = x.cuda().contiguous(memory_format=torch.channels_last)
+    for config in layernorm_2d_kernel_factory.configs(params, attr):
+        kernel = layernorm_2d_kernel_factory.make_kernel(params, config, attr)
+        kernel.compile()
+        kernel.load(0)
+        out = torch.full_like(xg, -42.0)
+        kernel(out, xg, w.cuda(), b.cuda())
+        torch.cuda.synchronize()
+        torch.testing.assert_close(out.float().cpu(), expected, rtol=2e-3, atol=4e-3, msg=str(config))
+        kernel.unload()
+
+
+def test_layer_and_backward():
+    torch.manual_seed(0)
+    layer = LayerNorm2d(96, eps=1e-6).cuda()
+    with torch.no_grad():
+        layer.weight.copy_(torch.randn(96))
+        layer.bias.copy_(torch.randn(96))
+    x = torch.randn(2, 96, 6, 5)
+    dy = torch.randn(2, 96, 6, 5)
+    xg = x.half().cuda().contiguous(memory_format=torch.channels_last).requires_grad_(True)
+    y = layer(xg)
+    y.backward(dy.half().cuda())
+    xr = x.half().float().requires_grad_(True)
+    wr = layer.weight.detach().cpu().clone().requires_grad_(True)
+    br = layer.bias.detach().cpu().clone().requires_grad_(True)
+    yr = _reference(xr, wr, br, 1e-6)
+    yr.backward(dy.half().float())
+    torch.testing.assert_close(y.float().cpu(), yr.detach(), rtol=2e-3, atol=4e-3)
+    torch.testing.assert_close(xg.grad.float().cpu(), xr.grad, rtol=4e-3, atol=4e-3)
+    torch.testing.assert_close(layer.weight.grad.cpu(), wr.grad, rtol=2e-3, atol=2e-2)
+    torch.testing.assert_close(layer.bias.grad.cpu(), br.grad, rtol=2e-3, atol=2e-2)
