@@ -77,6 +77,12 @@ def fused_backward_kernel(params: Conv2dGw8Params, device):
     return fused
 
 
+def reset_fused_backward_choices():
+    """Forget which shapes run the fused backward kernel (after the tuning records changed)."""
+    with _fused_choice_lock:
+        _fused_choice.clear()
+
+
 def _is_unit(value) -> bool:
     return value in (1, (1, 1))
 

@@ -42,6 +42,42 @@ class KernelSpec:
 
 
 
+class LaunchTimer:
+    """Times every Kernel.launch made while it is active, with HIP events on the launch stream.
+
+        with LaunchTimer() as timer:
+            model(x)
+        timer.averages(skip=2)   # {kernel: average microseconds, first 2 launches left out}
+
+    This is how kernels are timed in situ, inside a model with the cache state the model
+    produces (the reference reads the same from torch.profiler,
+    scripts/profile_block.py:646-701).
+    """
+
+    active = None
+
+    def __init__(self):
+        self.events = {}
+
+    def __enter__(self):
+        LaunchTimer.active = self
+        self.events = {}
+        return self
+
+    def __exit__(self, exc_type, exc_val, exc_tb):
+        LaunchTimer.active = None
+        return False
+
+    def averages(self, skip: int = 0):
+        """Average microseconds per launch of each kernel seen (after the first `skip`)."""
+        torch.cuda.synchronize()
+        out = {}
+        for kernel, pairs in self.events.items():
+            pairs = pairs[skip:] or pairs
+            out[kernel] = 1e3 * sum(a.elapsed_time(b) for a, b in pairs) / len(pairs)
+        return out
+
+
 class Kernel:
     """A compiled kernel bound to one device.  Made by KernelFactory.make_kernel."""
 
@@ -128,6 +164,12 @@ class Kernel:
             spec = self.kernel_spec
             lp = spec.launch_params
             stream = torch.cuda.current_stream(device).cuda_stream
+            timer = LaunchTimer.active
+            if timer is not None:
+                start = torch.cuda.Event(enable_timing=True)
+                stop = torch.cuda.Event(enable_timing=True)
+                timer.events.setdefault(self, []).append((start, stop))
+                start.record()
             if self.epilogue_function is None:
                 self.function.launch(lp.grid, lp.block, args, lp.shared_mem_bytes, stream)
             elif static_workspace:
@@ -142,6 +184,8 @@ class Kernel:
                 self.function.launch(lp.grid, lp.block, (workspace,) + args[1:], lp.shared_mem_bytes, stream)
                 ep = spec.epilogue_launch_params
                 self.epilogue_function.launch(ep.grid, ep.block, (args[0], workspace), ep.shared_mem_bytes, stream)
+            if timer is not None:
+                stop.record()
         except Exception as e:
             raise ValueError(f"Error in kernel {self}") from e
 

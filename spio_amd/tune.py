@@ -13,6 +13,7 @@ per shape instead of predicted.
 import argparse
 import os
 import sys
+from typing import Any, Dict, List, Optional, Sequence
 
 BENCH_SHAPES = [
     "32n_64c_56h_56w_1py_1px_3r_3s_nb",
@@ -27,6 +28,157 @@ NETWORK_SHAPES = [
     "128n_384c_14h_14w_1py_1px_3r_3s_b",
     "128n_768c_7h_7w_1py_1px_3r_3s_b",
 ]
+
+
+def tune_model(model, inputs: Sequence, backward: bool = True, max_configs: Optional[int] = 8,
+               iters: int = 5, warmup: int = 2, record_path: Optional[str] = None, record: bool = True,
+               autocast_dtype=None, loss=None) -> List[Dict[str, Any]]:  # fmt: skip
+    """Tune the kernels a model actually asks for, inside the model.
+
+    Takes the place of the reference's benchmarking harness (scripts/profile_block.py:545-701):
+      1. one forward (+ backward) pass under `KernelParamsLogger` records every
+         (kernel factory, params, kwargs) the model requests;
+      2. the candidate configurations of exactly those kernels are compiled (the `max_configs`
+         best-ranked ones of each; None = all);
+      3. round i pins the i-th candidate of every kernel through the caches' overlays
+         (`KernelCache.update_overlay`) and runs the model `warmup + iters` times over `inputs`
+         (a list of input batches, rotated) while `LaunchTimer` times each launch with HIP events:
+         kernels are timed with the cache state and neighbours they have in the model;
+      4. a round whose model output disagrees with the first round's is discarded as a whole
+         (one of its configurations computes something else);
+      5. the fastest candidate of every kernel is written to the tuning records (the user
+         record file, or `record_path`), the caches are cleared, and the next request for each
+         of these kernels compiles the recorded winner.
+
+    Returns one dict per kernel: name, chosen config, its microseconds, and all timed candidates.
+    """
+    import torch
+
+    from .compiler.compiler_pool import compile_kernel_configs
+    from .functional import reset_fused_backward_choices
+    from .hip import get_device_attributes
+    from .kernels.kernel import LaunchTimer
+    from .kernels.kernel_params_logger import KernelParamsLogger
+    from .kernels.tuner import config_to_dict, tuner
+
+    inputs = list(inputs) if isinstance(inputs, (list, tuple)) else [inputs]
+    if loss is None:
+        loss = lambda out: out.float().sum()  # noqa: E731
+
+    def run(x):
+        ctx = torch.autocast(device_type="cuda", dtype=autocast_dtype) if autocast_dtype else _NullContext()
+        if backward:
+            with ctx:
+                out = model(x)
+            loss(out).backward()
+            return out.detach()
+        with torch.no_grad(), ctx:
+            return model(x)
+
+    # 1. what does the model ask for?  (remembered fused/separate choices would hide requests)
+    reset_fused_backward_choices()
+    with KernelParamsLogger() as logger:
+        run(inputs[0])
+        torch.cuda.synchronize()
+    unique = list(dict.fromkeys(logger.get_logged_params()))
+    if not unique:
+        return []
+    caches = {id(kp.kernel_cache): kp.kernel_cache for kp in unique}
+    for cache in caches.values():
+        cache.clear_cache()
+    reset_fused_backward_choices()
+
+    # 2. candidates
+    table = {}
+    for kp in unique:
+        attr = get_device_attributes(kp.key.device_ordinal)
+        kwargs = dict(kp.kernel_kwargs)
+        configs = list(kp.kernel_factory.configs(kp.params, attr, **kwargs))
+        if max_configs is not None:
+            configs = configs[:max_configs]
+        table[kp] = compile_kernel_configs(kp.kernel_factory, kp.params, configs=configs, device_attr=attr, **kwargs)
+    rounds = max(len(kernels) for kernels in table.values())
+
+    # 3./4. rounds with pinned configurations.  Where the model's backward pass can run either the
+    # fused data+weight gradient kernel or the two separate ones, every round is run both ways so
+    # that all three families get their in-situ times.
+    times: Dict[Any, Dict[int, float]] = {kp: {} for kp in unique}
+    reference_out = None
+    discarded = []
+    has_fused = any(kp.kernel_factory.get_kernel_name(**dict(kp.kernel_kwargs)).endswith("bgrad") for kp in unique)
+    saved_mode = os.environ.get("SPIO_FUSED_BACKWARD")
+    passes = [(idx, mode) for idx in range(rounds) for mode in (("1", "0") if has_fused and backward else (None,))]
+    for idx, mode in passes:
+        if mode is not None:
+            os.environ["SPIO_FUSED_BACKWARD"] = mode
+        choice = {kp: kernels[idx % len(kernels)] for kp, kernels in table.items()}
+        overlays: Dict[int, Dict[Any, Any]] = {}
+        for kp, kernel in choice.items():
+            overlays.setdefault(id(kp.kernel_cache), {})[kp.key] = kernel
+            kernel.load(kp.key.device_ordinal, clear_code=False)
+        for cid, overlay in overlays.items():
+            caches[cid].update_overlay(overlay)
+        reset_fused_backward_choices()
+        try:
+            with LaunchTimer() as timer:
+                for i in range(warmup + iters):
+                    out = run(inputs[i % len(inputs)])
+                    if i == 0:
+                        first_out = out.float().clone()
+                averages = timer.averages(skip=warmup)
+        finally:
+            for cache in caches.values():
+                cache.clear_overlay()
+            for kernel in choice.values():
+                kernel.unload()
+            if mode is not None:
+                if saved_mode is None:
+                    os.environ.pop("SPIO_FUSED_BACKWARD", None)
+                else:
+                    os.environ["SPIO_FUSED_BACKWARD"] = saved_mode
+        if reference_out is None:
+            reference_out = first_out
+        elif not torch.allclose(first_out, reference_out, rtol=2e-2, atol=2e-2 * float(reference_out.abs().max())):
+            discarded.append((idx, mode))
+            continue
+        for kp, kernel in choice.items():
+            if idx < len(table[kp]) and kernel in averages:
+                times[kp][idx] = averages[kernel]
+
+    # 5. record the winners
+    results = []
+    for kp in unique:
+        kernels = table[kp]
+        attr = get_device_attributes(kp.key.device_ordinal)
+        kwargs = dict(kp.kernel_kwargs)
+        name = kp.kernel_factory.get_full_kernel_name(kp.params, **kwargs)
+        timed = sorted(times[kp].items(), key=lambda it: it[1])
+        entry = {"kernel": name, "candidates": len(kernels), "config": None, "us": None,
+                 "sweep": [{"config": config_to_dict(kernels[i].config), "us": us} for i, us in timed]}  # fmt: skip
+        if timed:
+            best_idx, best_us = timed[0]
+            entry["config"] = config_to_dict(kernels[best_idx].config)
+            entry["us"] = best_us
+            if record:
+                tuner._store(attr, name, {"config": entry["config"], "us": best_us, "candidates": len(kernels),
+                                          "sweep": entry["sweep"][:8], "in_situ": True}, record_path)  # fmt: skip
+        results.append(entry)
+        for kernel in kernels:
+            kernel.code = None
+    for cache in caches.values():
+        cache.clear_cache()
+    reset_fused_backward_choices()
+    if discarded:
+        print(f"spio: tune_model discarded rounds {discarded}: model output differed from the first round")
+    return results
+
+
+class _NullContext:
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
 
 
 def main(argv=None):
