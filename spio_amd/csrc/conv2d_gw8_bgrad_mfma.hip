@@ -405,12 +405,18 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
             const int h = p0 - 2 * kPadY + ts;
             const bool real = ts >= 2 * kPadY && ts < 2 * kPadY + bh_eff;
             const rsrc_t rs = real ? rs_dx : rs_none;
-            const int soff = __builtin_amdgcn_readfirstlane(imin(imax(h, 0), kH - 1) * ROW_BYTES);
+            // The row offset is added to the per-lane offset; the scalar-offset operand stays the
+            // constant 0.  A 16-byte buffer store reads its data registers for a few cycles after
+            // it issues, and only for the constant form does the compiler keep the next
+            // instructions from writing them: with the row offset in a scalar register a result
+            // moved into the first data register right behind the store was stored in its place
+            // (seen on gfx950 as stray values in the first two channels of some pixels).
+            const unsigned row_off = (unsigned)(imin(imax(h, 0), kH - 1) * ROW_BYTES);
 #pragma unroll
             for (int l = 0; l < LPTD; ++l) {
                 Pack16 v;
                 v.u = *reinterpret_cast<const spio_uint4*>(ostage + obuf * OUT_ROW_BYTES + o_lds[l]);
-                __builtin_amdgcn_raw_buffer_store_b128(v.i, rs, (int)d_voff[l], soff, AUX_NT);
+                __builtin_amdgcn_raw_buffer_store_b128(v.i, rs, (int)(d_voff[l] + row_off), 0, AUX_NT);
             }
         };
 

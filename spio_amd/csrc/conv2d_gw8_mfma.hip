@@ -107,18 +107,14 @@ constexpr int NBLKS = (kN + NB - 1) / NB;
 constexpr int NUM_BLOCKS = GBLKS * PBLKS * NBLKS;
 constexpr int STEPS = BP + kR - 1;
 
-constexpr int gcd_(int a, int b) { return b == 0 ? a : gcd_(b, a % b); }
-constexpr int LCM = NS / gcd_(NS, PF) * PF;  // lcm(NS, PF); even, so also a multiple of NR
-// Up to SPIO_MAX_UNROLL steps the whole step loop is unrolled (every rotation index and every
-// "is there a row to load / to store" is then a compile-time fact); longer loops run in chunks
-// of lcm(NS, PF) steps.
+// The step loop is unrolled completely: every rotation index and every "is there a row to load
+// / to store" is then a compile-time fact, and no memory instruction sits in a loop whose entry
+// and back edge would disagree about the operations in flight.
 #ifndef SPIO_MAX_UNROLL
 #define SPIO_MAX_UNROLL 64
 #endif
-constexpr bool kFullUnroll = STEPS <= SPIO_MAX_UNROLL;
-constexpr int CHUNK = kFullUnroll ? (STEPS + LCM - 1) / LCM * LCM : LCM;
-
-static_assert(PF >= 2 && WAVES <= 16 && LCM % NR == 0, "bad configuration");
+static_assert(STEPS <= SPIO_MAX_UNROLL, "block_p + R - 1 exceeds the unrolled step limit");
+static_assert(PF >= 2 && WAVES <= 16, "bad configuration");
 constexpr int STREAM_UNITS = NR * RING_ROW_UNITS + 2 * OUT_ROW_BYTES / 16;
 constexpr int FILTER_UNITS = kIgrad ? GB * 8 * kR * kS : 0;  // staged filters (data gradient only)
 constexpr int LDS_UNITS = STREAM_UNITS > FILTER_UNITS ? STREAM_UNITS : FILTER_UNITS;
@@ -409,129 +405,122 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
     }
 
     // ---- row 0 into the ring ----
-    block_sync();  // ring zeroed
+    block_sync();  // slack zeroed
 #pragma unroll
     for (int l = 0; l < LPT; ++l) ring[in_lds[l]] = pre[0][l];
     block_sync();
 
     // Coalesced store of the output row staged at step `ts` (in stage buffer `obuf`): the row
-    // that received its last tap at that step.  Called one step later, after the barrier.  Steps
-    // that finish no row, and rows past the end of the image, store through the empty
-    // descriptor: the instructions are issued all the same and the hardware drops them.
+    // that received its last tap at that step.  Called one step later, after the barrier.  Rows
+    // past the end of the image store through the empty descriptor: the instructions are issued
+    // all the same and the hardware drops them.
     auto store_output_row = [&](int ts, int obuf) {
         const int p = p0 + ts - (kR - 1);
-        const bool real = ts >= kR - 1 && p < DH;
-        const rsrc_t rs = real ? rs_dst : rs_dst_none;
-        const int soff = __builtin_amdgcn_readfirstlane(imin(imax(p, 0), DH - 1) * DST_ROW_BYTES);
+        const rsrc_t rs = p < DH ? rs_dst : rs_dst_none;
+        // The row offset is added to the per-lane offset; the scalar-offset operand stays the
+        // constant 0.  A 16-byte buffer store reads its data registers for a few cycles after it
+        // issues, and only for the constant form does the compiler keep the next instructions
+        // from writing them: with the row offset in a scalar register an accumulator moved into
+        // the first data register right behind the store was stored in its place (seen on gfx950
+        // as stray values in the first two channels of some pixels of one output row).
+        const unsigned row_off = (unsigned)(imin(imax(p, 0), DH - 1) * DST_ROW_BYTES);
 #pragma unroll
         for (int s = 0; s < SPT; ++s) {
             Pack16 v;
             v.u = *(lds_u4p)(ostage + obuf * OUT_ROW_BYTES + out_lds[s]);
-            __builtin_amdgcn_raw_buffer_store_b128(v.i, rs, (int)out_voff[s], soff, AUX_NT);
+            __builtin_amdgcn_raw_buffer_store_b128(v.i, rs, (int)(out_voff[s] + row_off), 0, AUX_NT);
         }
     };
 
-    for (int tb = 0; tb < STEPS; tb += CHUNK) {
+    // Rows above and below the image are rows of zeros in the ring; their products are skipped (a
+    // scalar branch around LDS reads and MFMAs only: with a 7-row filter on a 14-row image they
+    // would be 6 of 20 steps).
+    auto row_is_live = [&](int t) {
+        const int h = p0 + t - EPY;
+        return h >= 0 && h < SH;
+    };
+    spio_half8 bfrag[TPW][KB];
+    auto read_fragments = [&](spio_half8(&frag)[TPW][KB], int ring_row) {
+        const lds_u4p rrow = ring + ring_row * RING_ROW_UNITS + frag_unit;
 #pragma unroll
-        for (int uu = 0; uu < CHUNK; ++uu) {
-            const int t = tb + uu;
-            if (t >= STEPS) break;
-            const int ph = uu % NS;        // compile-time after unrolling
-            const int rbuf = uu % NR;      // ring row holding source row t
-            const int obuf = uu & 1;       // output stage buffer of this step
-            const int pbuf = uu % PF;      // register buffer that held row t
-
-            // 1. prefetch source row t+PF (its register buffer is free: row t is in LDS).  Past the
-            //    last row the chunked loop still issues its loads (through the empty descriptor), so
-            //    that every step has the same number of them; the unrolled loop leaves them out.
-            if (PF < STEPS && (!kFullUnroll || t + PF < STEPS)) {
-                if (t + PF < STEPS) {
-                    load_row(pre[pbuf], t + PF);
-                } else {
+        for (int i = 0; i < TPW; ++i) {
+            const int tile = ws + TS * i;
+            if (TS == 1 || tile < WT) {
 #pragma unroll
-                    for (int l = 0; l < LPT; ++l) {
-                        Pack16 v;
-                        v.i = __builtin_amdgcn_raw_buffer_load_b128(rs_src_none, (int)in_voff[l], 0, 0);
-                        pre[pbuf][l] = v.u;
-                    }
+                for (int u = 0; u < KB; ++u) {
+                    Pack16 v;
+                    v.u = rrow[16 * TS * i + 16 * ws + 4 * u];
+                    frag[i][u] = v.h;
                 }
             }
-
-            // 2. multiply source row t into the live output rows.  The fragment reads are issued
-            //    first; the previous step's output row is stored while they are in flight.  Rows
-            //    above and below the image are rows of zeros in the ring; their products are
-            //    skipped (a scalar branch around LDS reads and MFMAs only: with a 7-row filter on a
-            //    14-row image they would be 6 of 20 steps).
-            const int hcur = p0 + t - EPY;
-            const bool row_live = hcur >= 0 && hcur < SH;
-            spio_half8 bfrag[TPW][KB];
-            if (row_live) {
-                const lds_u4p rrow = ring + rbuf * RING_ROW_UNITS + frag_unit;
-#pragma unroll
-                for (int i = 0; i < TPW; ++i) {
-                    const int tile = ws + TS * i;
-                    if (TS == 1 || tile < WT) {
-#pragma unroll
-                        for (int u = 0; u < KB; ++u) {
-                            Pack16 v;
-                            v.u = rrow[16 * TS * i + 16 * ws + 4 * u];
-                            bfrag[i][u] = v.h;
-                        }
-                    }
-                }
-            }
-            if (!kFullUnroll || t >= kR) store_output_row(t - 1, (uu + 1) & 1);
-            if (row_live) {
-#pragma unroll
-                for (int i = 0; i < TPW; ++i) {
-                    const int tile = ws + TS * i;
-                    if (TS == 1 || tile < WT) {
-#pragma unroll
-                        for (int a = 0; a < NACC; ++a) {
-                            const int d = pmod(ph - 2 * a, NS);
-#pragma unroll
-                            for (int u = 0; u < KB; ++u)
-                                acc[i][a] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                                    wfrag[d][u], bfrag[i][u], acc[i][a], 0, 0, 0);
-                        }
-                    }
-                }
-            }
-
-            // 3. the row that received its last tap: stage it, reset its slot
-            {
-                const int slot = pmod(ph - (kR - 1), NS);
-                const int a = slot >> 1;
-                const int j = slot & 1;
-                const bool emit = t >= kR - 1;
-                if (out_j == j) {
-#pragma unroll
-                    for (int i = 0; i < TPW; ++i) {
-                        const int tile = ws + TS * i;
-                        if (TS == 1 || tile < WT) {
-                            if (emit) {
-                                Pack8 o;
-#pragma unroll
-                                for (int e = 0; e < 4; ++e) o.h[e] = (spio_half)acc[i][a][e];
-                                typedef __attribute__((address_space(3))) spio_uint2* lds_u2p;
-                                *(lds_u2p)(ostage_lane + obuf * OUT_ROW_BYTES + 16 * TS * i * OSTRIDE) = o.u;
-                            }
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) acc[i][a][e] = bias_reg[e];
-                        }
-                    }
-                }
-            }
-
-            // 4. source row t+1 (loaded earlier) into the other ring row
-            if (t + 1 < STEPS) {
-#pragma unroll
-                for (int l = 0; l < LPT; ++l)
-                    ring[((uu + 1) % NR) * RING_ROW_UNITS + in_lds[l]] = pre[(uu + 1) % PF][l];
-            }
-
-            block_sync();
         }
+    };
+#pragma unroll
+    for (int t = 0; t < STEPS; ++t) {
+        const int ph = t % NS;    // all of these are compile-time constants after unrolling
+        const int obuf = t & 1;   // output stage buffer of this step
+        const int pbuf = t % PF;  // register buffer that held row t
+
+        // 1. prefetch source row t+PF (its register buffer is free: row t is in LDS)
+        if (t + PF < STEPS) load_row(pre[pbuf], t + PF);
+
+        // 2. fragment reads of this step's row; the previous step's output row is stored while
+        //    they are in flight
+        const bool row_live = row_is_live(t);
+        if (row_live) read_fragments(bfrag, t % NR);
+        if (t >= kR) store_output_row(t - 1, (t + 1) & 1);
+
+        // 3. multiply source row t into the live output rows
+        if (row_live) {
+#pragma unroll
+            for (int i = 0; i < TPW; ++i) {
+                const int tile = ws + TS * i;
+                if (TS == 1 || tile < WT) {
+#pragma unroll
+                    for (int a = 0; a < NACC; ++a) {
+                        const int d = pmod(ph - 2 * a, NS);
+#pragma unroll
+                        for (int u = 0; u < KB; ++u)
+                            acc[i][a] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                wfrag[d][u], bfrag[i][u], acc[i][a], 0, 0, 0);
+                    }
+                }
+            }
+        }
+
+        // 4. the row that received its last tap: stage it, reset its slot
+        {
+            const int slot = pmod(ph - (kR - 1), NS);
+            const int a = slot >> 1;
+            const int j = slot & 1;
+            const bool emit = t >= kR - 1;
+            if (out_j == j) {
+#pragma unroll
+                for (int i = 0; i < TPW; ++i) {
+                    const int tile = ws + TS * i;
+                    if (TS == 1 || tile < WT) {
+                        if (emit) {
+                            Pack8 o;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) o.h[e] = (spio_half)acc[i][a][e];
+                            typedef __attribute__((address_space(3))) spio_uint2* lds_u2p;
+                            *(lds_u2p)(ostage_lane + obuf * OUT_ROW_BYTES + 16 * TS * i * OSTRIDE) = o.u;
+                        }
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[i][a][e] = bias_reg[e];
+                    }
+                }
+            }
+        }
+
+        // 5. the next source row not yet in the ring (loaded earlier) into its ring row
+        if (t + 1 < STEPS) {
+#pragma unroll
+            for (int l = 0; l < LPT; ++l)
+                ring[((t + 1) % NR) * RING_ROW_UNITS + in_lds[l]] = pre[(t + 1) % PF][l];
+        }
+
+        block_sync();
     }
     store_output_row(STEPS - 1, (STEPS - 1) & 1);  // the last row
 }

@@ -133,10 +133,6 @@ def _config_is_legal(params, config) -> bool:
         and g["REGISTERS"] <= MAX_REGISTERS
         and config.prefetch >= 2
         and config.prefetch % 2 == 0
-        # The chunked form of the step loop gave wrong grad_input values now and then in
-        # 16-wave workgroups (56-row blocks, lanes 12-15 of the 16-lane groups; cause not found;
-        # 8-wave workgroups and the unrolled form are clean in the same tests): not offered.
-        and (g["STEPS"] <= MAX_UNROLLED_STEPS or g["THREADS"] <= 512)
         and config.block_n * params.c * params.h * params.w * 2 < 2**31
     )
 

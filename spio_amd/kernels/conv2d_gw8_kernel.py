@@ -28,7 +28,7 @@ MAX_LDS_BYTES = 128 * 1024
 MAX_UNROLLED_STEPS = 64  # SPIO_MAX_UNROLL of the kernel: up to here the step loop is fully unrolled
 MAX_LOADS_PER_THREAD = 8
 MAX_ACCUMULATORS = 16
-MAX_CONFIGS = 32
+MAX_CONFIGS = 36
 PREFETCH_CHOICES = (2, 4, 8, 12, 16)
 MAX_GEOMETRIES = 24  # tile geometries that enter the sweep; the best few also try the other cache/XCD policies
 

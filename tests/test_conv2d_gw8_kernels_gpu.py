@@ -117,6 +117,22 @@ def test_fprop_explicit_configs():
                     configs=[Conv2dGw8Config(groups=8, block_p=8, block_n=1)])  # fmt: skip
 
 
+def test_stores_keep_their_data_registers():
+    """Configurations whose compiled code once wrote a result into the first data register of a
+    16-byte buffer store in the instruction behind it (row offset in a scalar register: no wait
+    state is inserted for that form), which now and then stored stray values in the first two
+    channels of some pixels of one output row.  Three runs each, full-size grids."""
+    params = Conv2dGw8Params(n=256, c=256, h=14, w=14, r=7, s=7, padding=3)
+    for seed in range(3):
+        run_kernel_test(conv2d_gw8_kernel_factory, params, seed=seed,
+                        configs=[Conv2dGw8Config(groups=4, block_p=14, block_n=2, prefetch=8),
+                                 Conv2dGw8Config(groups=4, block_p=14, block_n=2, prefetch=4)])  # fmt: skip
+    params = Conv2dGw8Params(n=8, c=64, h=56, w=56)
+    for seed in range(3):
+        run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params, seed=seed,
+                              configs=[Conv2dGw8BgradConfig(groups=8, block_h=0, prefetch=2, split=2)])  # fmt: skip
+
+
 @pytest.mark.slow
 @pytest.mark.parametrize("params", sample_params(seed=1), ids=lambda p: p.encode())
 def test_fprop_sampled(params):
