@@ -155,10 +155,12 @@ int spio_hip_launch_scratch(void* function,
                             void** params, int num_params,
                             int scratch_param, size_t scratch_bytes);
 
-/* Asynchronous fill of a device buffer with zero bytes on `stream`; used for
- * the pre-zeroed weight-gradient contract
- * (spio/functional/conv2d_gw8_function.py:124-127) by callers without torch. */
-int spio_hip_memset_zero_async(void* device_ptr, size_t bytes, void* stream);
+/* Asynchronous fill of a device buffer with zero bytes on `stream`, for the
+ * pre-zeroed weight-gradient contract
+ * (spio/functional/conv2d_gw8_function.py:124-127) by callers without torch.
+ * A fill kernel is launched, not a runtime memset, so the call may be recorded
+ * under HIP graph capture like any other kernel launch. */
+int spio_hip_zero_fill_async(void* device_ptr, size_t bytes, void* stream);
 
 /* Replace get_device_attributes, ctx_synchronize, get_driver_version
  * (driver.pyx:284-303, 360-369) and PrimaryContextGuard.set_device (259-265). */

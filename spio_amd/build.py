@@ -1,9 +1,10 @@
 """Builds the native pieces of the package in-tree.
 
 `build_native()` builds csrc/libspio_hip.so from csrc/spio_hip.cpp (host C++;
-it binds the HIP runtime and hipRTC with dlopen) and csrc/spio_hip_scratch.hip
-(hipcc, gfx950: the static device workspace and the launch that uses it, which
-links the HIP runtime by its soname, so the copy a host framework has already
+it binds the HIP runtime and hipRTC with dlopen) and the device sources
+csrc/spio_hip_scratch.hip and csrc/spio_hip_fill.hip (hipcc, gfx950: the static
+device workspace with the launch that uses it, and the zero-fill kernel; they
+link the HIP runtime by its soname, so the copy a host framework has already
 mapped is the one used).  hipcc cross-compiles, so this builds on machines
 without a GPU.
 
@@ -22,6 +23,9 @@ CSRC_DIR = os.path.join(_HERE, "csrc")
 REPO_INCLUDE_DIR = os.path.join(os.path.dirname(_HERE), "include")
 LIB_PATH = os.path.join(CSRC_DIR, "libspio_hip.so")
 ROCM_HOME = os.environ.get("ROCM_PATH") or os.environ.get("ROCM_HOME") or "/opt/rocm"
+
+# Device translation units of libspio_hip.so.
+DEVICE_SOURCES = ["spio_hip_scratch.hip", "spio_hip_fill.hip"]
 
 # hipcc flags shared by every device compilation of this package.
 HIPCC_DEVICE_FLAGS = [
@@ -53,8 +57,8 @@ def _run(cmd, what, verbose=False):
 def build_native(force: bool = True, verbose: bool = False) -> str:
     """Compile libspio_hip.so; returns its path."""
     host_src = os.path.join(CSRC_DIR, "spio_hip.cpp")
-    dev_src = os.path.join(CSRC_DIR, "spio_hip_scratch.hip")
-    deps = [host_src, dev_src, os.path.join(CSRC_DIR, "spio_hip_internal.h"),
+    dev_srcs = [os.path.join(CSRC_DIR, name) for name in DEVICE_SOURCES]
+    deps = [host_src, *dev_srcs, os.path.join(CSRC_DIR, "spio_hip_internal.h"),
             os.path.join(_include_dir(), "spio_hip.h")]  # fmt: skip
     if not force and os.path.exists(LIB_PATH) and all(
         os.path.getmtime(LIB_PATH) >= os.path.getmtime(d) for d in deps
@@ -67,18 +71,19 @@ def build_native(force: bool = True, verbose: bool = False) -> str:
     includes = [f"-I{_include_dir()}", f"-I{CSRC_DIR}", f"-I{os.path.join(ROCM_HOME, 'include')}"]
     tag = f".tmp{os.getpid()}"
     host_obj = os.path.join(CSRC_DIR, f"spio_hip{tag}.o")
-    dev_obj = os.path.join(CSRC_DIR, f"spio_hip_scratch{tag}.o")
+    dev_objs = [os.path.splitext(src)[0] + f"{tag}.o" for src in dev_srcs]
     tmp = LIB_PATH + tag
     try:
         _run([cxx, "-O2", "-std=c++17", "-fPIC", "-Wall", "-fvisibility-inlines-hidden", *includes,
               "-c", "-o", host_obj, host_src], "compiling spio_hip.cpp", verbose)  # fmt: skip
-        _run([hipcc, *HIPCC_DEVICE_FLAGS, "-fPIC", *includes, "-c", "-o", dev_obj, dev_src],
-             "compiling spio_hip_scratch.hip", verbose)  # fmt: skip
-        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, host_obj, dev_obj,
+        for src, obj in zip(dev_srcs, dev_objs):
+            _run([hipcc, *HIPCC_DEVICE_FLAGS, "-fPIC", *includes, "-c", "-o", obj, src],
+                 f"compiling {os.path.basename(src)}", verbose)  # fmt: skip
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, host_obj, *dev_objs,
               "-ldl", "-lpthread"], "linking libspio_hip.so", verbose)  # fmt: skip
         os.replace(tmp, LIB_PATH)
     finally:
-        for f in (host_obj, dev_obj, tmp):
+        for f in (host_obj, *dev_objs, tmp):
             if os.path.exists(f):
                 os.remove(f)
     return LIB_PATH

@@ -65,7 +65,6 @@ struct Api {
     hipError_t (*hipEventRecord)(hipEvent_t, hipStream_t) = nullptr;
     hipError_t (*hipEventSynchronize)(hipEvent_t) = nullptr;
     hipError_t (*hipEventElapsedTime)(float*, hipEvent_t, hipEvent_t) = nullptr;
-    hipError_t (*hipMemsetAsync)(void*, int, size_t, hipStream_t) = nullptr;
     const char* (*hipGetErrorString)(hipError_t) = nullptr;
 
     hiprtcResult (*hiprtcCreateProgram)(hiprtcProgram*, const char*, const char*, int,
@@ -193,7 +192,6 @@ int spio_hip_init(const char* hip_library_path, const char* hiprtc_library_path)
     bind(h, "hipEventRecord", &api.hipEventRecord, &missing);
     bind(h, "hipEventSynchronize", &api.hipEventSynchronize, &missing);
     bind(h, "hipEventElapsedTime", &api.hipEventElapsedTime, &missing);
-    bind(h, "hipMemsetAsync", &api.hipMemsetAsync, &missing);
     bind(h, "hipGetErrorString", &api.hipGetErrorString, &missing);
     void* r = api.rtc_handle;
     bind(r, "hiprtcCreateProgram", &api.hiprtcCreateProgram, &missing);
@@ -429,14 +427,6 @@ int spio_hip_launch_sequence_timed(const spio_hip_launch_desc_t* descs, int stag
     (void)g_api.hipEventDestroy(start);
     (void)g_api.hipEventDestroy(stop);
     if (e != hipSuccess) return hip_fail(e, "timed launch sequence");
-    return SPIO_HIP_OK;
-}
-
-int spio_hip_memset_zero_async(void* device_ptr, size_t bytes, void* stream) {
-    REQUIRE_READY();
-    if (!device_ptr && bytes) return fail(SPIO_HIP_ERR_ARGUMENT, "memset: null pointer");
-    if (!bytes) return SPIO_HIP_OK;
-    HIP_TRY(hipMemsetAsync(device_ptr, 0, bytes, static_cast<hipStream_t>(stream)));
     return SPIO_HIP_OK;
 }
 

@@ -21,6 +21,6 @@ from .driver import (
     synchronize,
     stream_synchronize,
     set_device,
-    memset_zero_async,
+    zero_fill_async,
     launch_sequence_timed,
 )

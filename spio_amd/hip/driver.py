@@ -105,7 +105,7 @@ _SIGNATURES = {
          ctypes.POINTER(ctypes.c_float)],
         ctypes.c_int,
     ),
-    "spio_hip_memset_zero_async": ([_vp, ctypes.c_size_t, _vp], ctypes.c_int),
+    "spio_hip_zero_fill_async": ([_vp, ctypes.c_size_t, _vp], ctypes.c_int),
     "spio_hip_device_count": ([ctypes.POINTER(ctypes.c_int)], ctypes.c_int),
     "spio_hip_device_attrs": ([ctypes.c_int, ctypes.POINTER(_DeviceAttrsStruct)], ctypes.c_int),
     "spio_hip_set_device": ([ctypes.c_int], ctypes.c_int),
@@ -504,7 +504,8 @@ def stream_synchronize(stream: int = 0):
     _check(_lib.spio_hip_stream_synchronize(stream or None))
 
 
-def memset_zero_async(ptr: int, nbytes: int, stream: int = 0):
-    """Zero `nbytes` of device memory asynchronously on `stream`."""
+def zero_fill_async(ptr: int, nbytes: int, stream: int = 0):
+    """Zero `nbytes` of device memory asynchronously on `stream` with a fill kernel (any
+    alignment, any size; safe to record under HIP graph capture)."""
     init()
-    _check(_lib.spio_hip_memset_zero_async(ptr, nbytes, stream or None))
+    _check(_lib.spio_hip_zero_fill_async(ptr, nbytes, stream or None))

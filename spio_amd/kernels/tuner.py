@@ -30,6 +30,7 @@ import dataclasses
 import json
 import os
 import threading
+import sys
 import time
 from typing import Any, Dict, List, Optional
 
@@ -169,6 +170,11 @@ class Tuner:
             if not configs:
                 raise ValueError(f"no kernel configuration supports {params}")
             name = kernel_factory.get_full_kernel_name(params, **kernel_kwargs)
+            if all(getattr(c, "variant", "mfma") == "direct" for c in configs):
+                # not an error, but a cliff the user should hear about: no MFMA tiling fits
+                # (registers, LDS or the unrolled-step limit), the any-shape kernel runs
+                print(f"spio: {name}: no MFMA configuration fits this shape; the any-shape kernel "
+                      "is used and runs at a fraction of the MFMA kernels' throughput", file=sys.stderr)  # fmt: skip
             mode = _mode()
             record = None if mode == "force" else self.lookup(device_attr, name)
             if record is not None:

@@ -3,6 +3,7 @@ geometry, JIT specialisation of every kernel family, caches and the tuner's
 record store.  CPU only."""
 
 import json
+import os
 
 import pytest
 
@@ -51,6 +52,47 @@ def test_every_shape_has_legal_configs(igrad):
             spec = conv2d_gw8_kernel_factory.get_kernel_spec(params, cfg, ATTR, igrad=igrad)
             assert spec.launch_params.grid[0] == g["NUM_BLOCKS"]
             assert spec.launch_params.block[0] == g["THREADS"]
+
+
+def test_model_shapes_and_wide_rows_get_mfma_kernels(capsys):
+    """No performance cliff onto the any-shape kernel: every model-derived shape (at its full
+    batch) and rows up to 128 pixels wide have an MFMA configuration in every family, and a
+    shape that has none (here: a row too wide for the LDS ring) says so on first use."""
+    from helpers import GOLDEN
+
+    with open(os.path.join(GOLDEN, "conv2d_gw8_model_shapes.json"), encoding="utf-8") as f:
+        rows = json.load(f)
+    shapes = [Conv2dGw8Params(n=d["n"], c=d["c"], h=d["h"], w=d["w"], padding=(d["py"], d["px"]),
+                              r=d["r"], s=d["s"], has_bias=d["has_bias"]) for d in rows]  # fmt: skip
+    shapes += [Conv2dGw8Params(n=8, c=c, h=64, w=w) for c in (64, 256) for w in (64, 96, 128)]
+    shapes += [Conv2dGw8Params(n=8, c=256, h=64, w=64, r=7, s=7, padding=3)]
+    for params in shapes:
+        for factory, kw in ((conv2d_gw8_kernel_factory, {}), (conv2d_gw8_kernel_factory, {"igrad": True}),
+                            (conv2d_gw8_wgrad_kernel_factory, {})):  # fmt: skip
+            configs = factory.configs(params, ATTR, **kw)
+            assert any(c.variant == "mfma" for c in configs), f"{factory.get_full_kernel_name(params, **kw)}: direct only"
+
+    # the cliff is announced where it remains
+    huge = Conv2dGw8Params(n=1, c=64, h=8, w=4000)
+    configs = conv2d_gw8_kernel_factory.configs(huge, ATTR)
+    assert [c.variant for c in configs] == ["direct"]
+
+    class Stop(Exception):
+        pass
+
+    def no_compile(*a, **k):
+        raise Stop
+
+    import spio_amd.kernels.kernel_cache as kernel_cache
+
+    saved = kernel_cache.compile_and_load_kernel
+    kernel_cache.compile_and_load_kernel = no_compile
+    try:
+        with pytest.raises(Stop):
+            Tuner().best_kernel(conv2d_gw8_kernel_factory, huge, 0, ATTR)
+    finally:
+        kernel_cache.compile_and_load_kernel = saved
+    assert "no MFMA configuration fits" in capsys.readouterr().err
 
 
 def test_kernel_names_follow_the_reference_convention():
