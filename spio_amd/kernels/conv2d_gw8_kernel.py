@@ -4,7 +4,9 @@ Reference: spio/kernels/conv2d_gw8_kernel.py:30-238 (`Conv2dGw8Config`,
 `_get_configs`, `_get_kernel_spec`; `igrad=True` selects the data gradient,
 which reuses the forward kernel with the flipped, group-transposed filter and
 padding (R-1-py, S-1-px), :73-83).  The tile configuration is re-designed for
-CDNA4: see csrc/conv2d_gw8_mfma.hip for what the fields mean on the device.
+CDNA4: see csrc/conv2d_gw8_mfma.hip (row-streaming kernel) and
+csrc/conv2d_gw8_image_mfma.hip (whole-image kernel for small images) for what
+the fields mean on the device.
 """
 
 from dataclasses import dataclass, replace
@@ -21,6 +23,7 @@ from .kernel_factory import KernelFactory
 from .launch_params import LaunchParams
 
 MFMA_SOURCE = "conv2d_gw8_mfma.hip"
+IMAGE_SOURCE = "conv2d_gw8_image_mfma.hip"
 DIRECT_SOURCE = "conv2d_gw8_direct.hip"
 
 MAX_WAVES = 16
@@ -29,6 +32,8 @@ MAX_UNROLLED_STEPS = 64  # SPIO_MAX_UNROLL of the kernel: up to here the step lo
 MAX_LOADS_PER_THREAD = 8
 MAX_ACCUMULATORS = 16
 MAX_CONFIGS = 36
+DEVICE_LDS_BYTES = 160 * 1024
+MAX_IMAGE_CONFIGS = 8  # whole-image configurations that enter the sweep
 PREFETCH_CHOICES = (2, 4, 8, 12, 16)
 MAX_GEOMETRIES = 24  # tile geometries that enter the sweep; the best few also try the other cache/XCD policies
 
@@ -49,8 +54,14 @@ class Conv2dGw8Config:
         xcd_chunk: consecutive tiles that go to the same XCD (they share halo rows through its
             L2) before the next run of tiles goes to the next XCD; 0 = one contiguous range of
             tiles per XCD, 1 = tiles dealt round-robin.
-        variant: "mfma" (row-streaming MFMA kernel) or "direct" (one thread per
-            output pixel-group; any shape).
+        block_n_iters: whole-image kernel only: image blocks a workgroup processes one after
+            the other with the same filter fragments.
+        variant: "mfma" (row-streaming MFMA kernel), "image" (whole-image MFMA kernel: image
+            blocks of block_n images move through LDS whole, `split` waves share a group by
+            splitting its accumulators; prefetch = 2 means two LDS buffers each for input and
+            output, prefetch = 1 one of each, which lets two workgroups share a CU; block_p and
+            the cache/XCD policies do not apply) or "direct" (one thread per output
+            pixel-group; any shape).
     """
 
     groups: int = 8
@@ -62,6 +73,7 @@ class Conv2dGw8Config:
     nontemporal: int = 1
     halo_cached: int = 1
     xcd_chunk: int = 4
+    block_n_iters: int = 1
 
 
 def direction_geometry(params: Conv2dGw8Params, igrad: bool) -> Dict[str, int]:
@@ -99,6 +111,101 @@ def mfma_geometry(params: Conv2dGw8Params, config: Conv2dGw8Config, igrad: bool)
     )  # fmt: skip
     d["NUM_BLOCKS"] = d["GBLKS"] * d["PBLKS"] * d["NBLKS"]
     return d
+
+
+def image_geometry(params: Conv2dGw8Params, config: Conv2dGw8Config, igrad: bool) -> Dict[str, int]:
+    """Host mirror of the compile-time constants of conv2d_gw8_image_mfma.hip."""
+    d = direction_geometry(params, igrad)
+    r, s = params.r, params.s
+    gb, nb, ts, iters = config.groups, config.block_n, config.split, config.block_n_iters
+    ns = 2 * ((r + 1) // 2)
+    nacc = ns // 2
+    kb = (s + 3) // 4
+    wpi = d["DW"] + s - 1
+    f = nb * wpi
+    wt = divup(f - s + 1, 16)
+    fp = 16 * wt + 4 * kb - 1
+    gs = fp + ((9 - fp % 16) + 16) % 16
+    threads = 64 * gb * ts
+    nbuf = 2 if config.prefetch >= 2 else 1  # prefetch = 1: single buffers (SPIO_DB = 0)
+    in_units = d["SH"] * gb * gs
+    out_bytes = d["DH"] * 16 * wt * (gb * 16 + 16)
+    # input buffers, dump cells, output buffers (which first hold the groups' filters)
+    lds = (nbuf * in_units + 32) * 16 + max(nbuf * out_bytes, gb * 8 * r * s * 16)
+    lpt = divup(d["SH"] * nb * d["SW"] * gb, threads)
+    spt = divup(d["DH"] * nb * d["DW"] * gb, threads)
+    wlpt = divup(gb * 8 * r * s, threads)
+    apw = max(nacc // max(ts, 1), 1)
+    d.update(
+        NS=ns, NACC=nacc, APW=apw, KB=kb, WPI=wpi, F=f, WT=wt, GS=gs, THREADS=threads,
+        LDS_BYTES=lds, LPT=lpt, SPT=spt, STEPS=d["DH"] + r - 1,
+        GBLKS=divup(params.groups, gb), NBLKS=divup(params.n, nb),
+        # filter fragments, accumulators, source fragments, block in flight, addressing, the rest
+        REGISTERS=4 * ns * kb + 4 * wt * apw + 8 * wt * kb + 4 * max(2 * lpt, lpt + wlpt) + 2 * (lpt + spt) + 14,
+        NBUF=nbuf,
+    )  # fmt: skip
+    d["WGBLKS"] = divup(d["NBLKS"], iters)
+    d["NUM_BLOCKS"] = d["GBLKS"] * d["WGBLKS"]
+    return d
+
+
+def _image_config_is_legal(params, config, igrad) -> bool:
+    g = image_geometry(params, config, igrad)
+    waves = config.groups * config.split
+    return (
+        waves <= MAX_WAVES
+        and config.split >= 1
+        and g["NACC"] % config.split == 0
+        and config.block_n <= max(params.n, 1)
+        and config.block_n_iters >= 1
+        and g["LDS_BYTES"] <= DEVICE_LDS_BYTES
+        and g["LPT"] <= MAX_LOADS_PER_THREAD
+        and g["SPT"] <= MAX_LOADS_PER_THREAD
+        and g["STEPS"] <= MAX_UNROLLED_STEPS
+        # registers per lane: 128 where a SIMD must hold four waves of the workgroup, else 256
+        and g["REGISTERS"] <= (128 if waves > 8 else 232)
+        and config.block_n * params.c * max(params.h * params.w, params.p * params.q) * 2 < 2**31
+    )
+
+
+def _image_score(params, config, igrad, num_cus: int) -> float:
+    """Relative cost of a whole-image configuration; lower is better.  Prices idle compute units
+    (grid quantisation; LDS decides how many workgroups a CU holds), wasted MFMA columns, partial
+    128-byte lines, the set-up a workgroup pays before its first block (filters through LDS,
+    pipeline fill: about two blocks' worth, measured) and, weakly, split accumulators."""
+    g = image_geometry(params, config, igrad)
+    per_cu = max(1, min(DEVICE_LDS_BYTES // g["LDS_BYTES"], 2048 // g["THREADS"]))
+    slots = num_cus * per_cu
+    rounds = divup(g["NUM_BLOCKS"], slots)
+    quant = rounds * slots / g["NUM_BLOCKS"]
+    tile_eff = config.block_n * g["DW"] / (16.0 * g["WT"])
+    group_eff = params.groups / (g["GBLKS"] * config.groups)
+    split_line = 1.0 if (config.groups * 16) % 128 == 0 or config.groups == params.groups else 1.2
+    setup = 1.0 + 2.0 / config.block_n_iters
+    split = 1.0 + 0.05 * (config.split - 1)
+    single = 1.0 if config.prefetch >= 2 else 1.03
+    ragged = g["WGBLKS"] * config.block_n_iters * config.block_n / params.n
+    return quant * ragged * split_line * setup * split * single / (tile_eff * group_eff)
+
+
+def _image_configs(params: Conv2dGw8Params, igrad: bool, num_cus: int) -> List[Conv2dGw8Config]:
+    """Legal whole-image configurations, most promising first (none for large images)."""
+    G = params.groups
+    found = []
+    for gb in sorted({g for g in (4, 8, 16, G) if g <= min(G, MAX_WAVES)}):
+        for nb in (1, 2, 4, 8):
+            for ts in (1, 2, 4):
+                for iters in (1, 2, 4, 8, 16):
+                    for buffers in (2, 1):
+                        cfg = Conv2dGw8Config(groups=gb, block_p=direction_geometry(params, igrad)["DH"],
+                                              block_n=nb, split=ts, prefetch=buffers, variant="image",
+                                              halo_cached=0, xcd_chunk=0, block_n_iters=iters)  # fmt: skip
+                        if nb * iters > max(params.n, 1) and iters > 1:
+                            continue
+                        if _image_config_is_legal(params, cfg, igrad):
+                            found.append((_image_score(params, cfg, igrad, num_cus), cfg))
+    found.sort(key=lambda sc: sc[0])
+    return [cfg for _, cfg in found[:MAX_IMAGE_CONFIGS]]
 
 
 def _mfma_config_is_legal(params, config, igrad) -> bool:
@@ -181,6 +288,10 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None, igrad: bool = False)
         for hc, ch in ((0, 4), (1, 0), (0, 0)):
             configs.append(replace(cfg, halo_cached=hc, xcd_chunk=ch))
     configs = configs[:MAX_CONFIGS]
+    # small images: the whole-image kernel; its two best candidates go first, so that the capped
+    # sweep an operator runs on an unrecorded shape sees both kernels
+    image = _image_configs(params, igrad, num_cus)
+    configs = image[:2] + configs + image[2:]
     configs.append(Conv2dGw8Config(groups=1, block_p=1, block_n=1, split=1, variant="direct"))
     return configs
 
@@ -206,6 +317,17 @@ def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8Config, _device_a
         defines["SPIO_BLOCK_THREADS"] = threads
         total = params.n * d["DH"] * d["DW"] * params.groups
         return KernelSpec(defines, LaunchParams(grid=divup(total, threads), block=threads), DIRECT_SOURCE)
+    if config.variant == "image":
+        assert _image_config_is_legal(params, config, igrad), f"illegal configuration {config} for {params}"
+        g = image_geometry(params, config, igrad)
+        defines.update(
+            SPIO_GB=config.groups, SPIO_NB=config.block_n, SPIO_TS=config.split,
+            SPIO_ITERS=config.block_n_iters, SPIO_NT=config.nontemporal,
+            SPIO_DB=int(config.prefetch >= 2),
+        )  # fmt: skip
+        return KernelSpec(
+            defines, LaunchParams(grid=g["NUM_BLOCKS"], block=g["THREADS"]), IMAGE_SOURCE, notes=g
+        )
     if config.variant != "mfma":
         raise ValueError(f"unknown kernel variant {config.variant!r}")
     assert _mfma_config_is_legal(params, config, igrad), f"illegal configuration {config} for {params}"

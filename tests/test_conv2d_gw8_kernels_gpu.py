@@ -117,6 +117,38 @@ def test_fprop_explicit_configs():
                     configs=[Conv2dGw8Config(groups=8, block_p=8, block_n=1)])  # fmt: skip
 
 
+def _image(groups, block_n, split, iters, buffers=2):
+    return Conv2dGw8Config(groups=groups, block_p=0, block_n=block_n, split=split, prefetch=buffers,
+                           variant="image", block_n_iters=iters, halo_cached=0, xcd_chunk=0)  # fmt: skip
+
+
+IMAGE_CASES = [
+    # 7x7 filter on 14x14: accumulators split over 1, 2, 4 waves; 1..4 image blocks per workgroup;
+    # a batch that does not fill the last workgroup's blocks
+    (Conv2dGw8Params(n=7, c=64, h=14, w=14, r=7, s=7, padding=3),
+     [_image(8, 1, 1, 1), _image(8, 1, 1, 5), _image(4, 1, 4, 2), _image(4, 1, 2, 3, 1), _image(4, 1, 2, 16),
+      _image(8, 1, 1, 2, 1), _image(4, 2, 2, 3, 1)]),
+    # 3x3 with a bias, images side by side, a group count that leaves idle waves (5 groups, 4 per block)
+    (Conv2dGw8Params(n=9, c=40, h=14, w=14, has_bias=True),
+     [_image(4, 2, 1, 2), _image(4, 1, 2, 1, 1), _image(5, 1, 1, 4), _image(2, 4, 2, 1), _image(5, 2, 1, 3, 1)]),
+    # 7x7 images
+    (Conv2dGw8Params(n=12, c=64, h=7, w=7, has_bias=True), [_image(8, 2, 1, 2), _image(8, 2, 2, 1), _image(4, 4, 1, 3), _image(8, 4, 1, 3, 1)]),
+    # 5x5 (three accumulators: splits 1 and 3), non-square image
+    (Conv2dGw8Params(n=5, c=32, h=9, w=12, r=5, s=5, padding=2, has_bias=True), [_image(4, 1, 3, 2), _image(4, 2, 1, 2, 1)]),
+    # asymmetric filter and padding, output larger than the input (the data gradient then crops)
+    (Conv2dGw8Params(n=3, c=16, h=6, w=8, r=3, s=3, padding=2), [_image(2, 1, 1, 2), _image(2, 2, 2, 1), _image(2, 1, 1, 3, 1)]),
+    (Conv2dGw8Params(n=4, c=16, h=10, w=6, r=4, s=1, padding=(2, 0), has_bias=True), [_image(2, 2, 2, 2)]),
+    (Conv2dGw8Params(n=2, c=16, h=8, w=8, r=3, s=3, padding=0), [_image(2, 1, 1, 2)]),
+]
+
+
+@pytest.mark.parametrize("params,configs", IMAGE_CASES, ids=lambda v: v.encode() if hasattr(v, "encode") else "")
+def test_whole_image_kernel_configs(params, configs):
+    """The whole-image forward / data-gradient kernel over explicit configurations."""
+    run_kernel_test(conv2d_gw8_kernel_factory, params, configs=configs)
+    run_grad_kernel_test(conv2d_gw8_kernel_factory, params, configs=configs, igrad=True)
+
+
 def test_stores_keep_their_data_registers():
     """Configurations whose compiled code once wrote a result into the first data register of a
     16-byte buffer store in the instruction behind it (row offset in a scalar register: no wait

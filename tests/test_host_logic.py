@@ -21,7 +21,7 @@ from spio_amd.kernels import (
     conv2d_gw8_wgrad_kernel_factory,
     kernel_params_logging_is_enabled,
 )
-from spio_amd.kernels.conv2d_gw8_kernel import MAX_LDS_BYTES, mfma_geometry
+from spio_amd.kernels.conv2d_gw8_kernel import MAX_LDS_BYTES, image_geometry, mfma_geometry
 from spio_amd.kernels.tuner import Tuner, device_key
 
 ATTR = DeviceAttributes()
@@ -45,6 +45,14 @@ def test_every_shape_has_legal_configs(igrad):
         assert configs and configs[-1].variant == "direct"
         assert len(set(configs)) == len(configs)
         for cfg in configs[:-1]:
+            if cfg.variant == "image":  # the whole-image kernel has its own geometry
+                g = image_geometry(params, cfg, igrad)
+                assert g["THREADS"] <= 1024 and g["LDS_BYTES"] <= 160 * 1024 and g["NACC"] % cfg.split == 0
+                spec = conv2d_gw8_kernel_factory.get_kernel_spec(params, cfg, ATTR, igrad=igrad)
+                assert spec.launch_params.grid[0] == g["NUM_BLOCKS"] == g["GBLKS"] * g["WGBLKS"]
+                assert spec.launch_params.block[0] == g["THREADS"]
+                assert g["WGBLKS"] * cfg.block_n_iters * cfg.block_n >= params.n
+                continue
             g = mfma_geometry(params, cfg, igrad)
             assert g["THREADS"] <= 1024 and g["LDS_BYTES"] <= MAX_LDS_BYTES
             assert g["NUM_BLOCKS"] >= 1 and g["WT"] * 16 >= g["F"] - params.s + 1
