@@ -185,6 +185,20 @@ SPIO_DEVICE void run(spio_uint4* __restrict__ dst, const spio_uint4* __restrict_
     const int gglob = cb * GB + wg;
     const bool wave_active = gglob < kGroups;  // idle waves compute on zeros and store nothing
 
+    // ---- the filters first: everything up to the first multiplication waits for them (global
+    //      memory -> LDS -> barrier -> fragments), the image blocks are not needed before ----
+    // the workgroup's filters as they lie in memory ([group][k or jj][r][s][8 ch]), coalesced
+    spio_uint4 wraw[WLPT];
+#pragma unroll
+    for (int l = 0; l < WLPT; ++l) {
+        const int i = imin(tid + THREADS * l, FILTER_UNITS - 1);
+        const int g = i / (8 * kR * kS);
+        const int rem = i % (8 * kR * kS);
+        const int gs = cb * GB + g < kGroups ? cb * GB + g : 0;
+        wraw[l] = reinterpret_cast<const spio_uint4*>(weights)[(long long)gs * (8 * kR * kS) + rem];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
     // ---- loop-invariant addressing of the cooperative block load and store ----
     unsigned in_voff[LPT];  // byte offset inside the image block
     int in_lds[LPT];        // 16-byte unit inside an input buffer
@@ -255,23 +269,13 @@ SPIO_DEVICE void run(spio_uint4* __restrict__ dst, const spio_uint4* __restrict_
         }
     };
 
-    // ---- first block and the filters on their way ----
+    // ---- the first two blocks on their way ----
     // Two register sets hold the blocks in flight: at any time the loads of two image blocks per
     // workgroup are outstanding (one block per CU does not cover the memory latency: each phase
     // would wait for its block, and the device would run at a fraction of its bandwidth).
     spio_uint4 pre0[LPT], pre1[LPT];
     load_block(pre0, first_blk, true);
     load_block(pre1, first_blk + 1, ITERS > 1);
-    // the workgroup's filters as they lie in memory ([group][k or jj][r][s][8 ch]), coalesced
-    spio_uint4 wraw[WLPT];
-#pragma unroll
-    for (int l = 0; l < WLPT; ++l) {
-        const int i = imin(tid + THREADS * l, FILTER_UNITS - 1);
-        const int g = i / (8 * kR * kS);
-        const int rem = i % (8 * kR * kS);
-        const int gs = cb * GB + g < kGroups ? cb * GB + g : 0;
-        wraw[l] = reinterpret_cast<const spio_uint4*>(weights)[(long long)gs * (8 * kR * kS) + rem];
-    }
     __builtin_amdgcn_sched_barrier(0);  // both requests leave before anything waits
 
     // ---- while they travel: clear the input buffers (halo columns and slack stay zero from
