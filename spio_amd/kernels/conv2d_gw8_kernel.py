@@ -291,7 +291,10 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None, igrad: bool = False)
     # small images: the whole-image kernel; its two best candidates go first, so that the capped
     # sweep an operator runs on an unrecorded shape sees both kernels
     image = _image_configs(params, igrad, num_cus)
-    configs = image[:2] + configs + image[2:]
+    if image and image_geometry(params, image[0], igrad)["NUM_BLOCKS"] >= num_cus:
+        configs = image[:2] + configs + image[2:]
+    else:  # too few image blocks to fill the device with workgroups that each pay the set-up
+        configs = configs[:2] + image[:2] + configs[2:] + image[2:]
     configs.append(Conv2dGw8Config(groups=1, block_p=1, block_n=1, split=1, variant="direct"))
     return configs
 
