@@ -121,7 +121,12 @@ constexpr int CPW = (KC + TS - 1) / TS;      // 32-pixel chunks per wave
 // group, (atomic publishing) every group's R*S*64 sums in grad_weight order, and eight
 // grad_bias sums per wave.
 constexpr int RING_UNITS = NRX * XROW_UNITS + NRD * DROW_UNITS;
-constexpr int SCRATCH_FLOATS = NBLK * 128;  // per wave
+// Filter rows whose row-slot halves are exchanged through the per-wave scratch in one go: all of
+// them where that fits 96 KB of LDS for the workgroup (every exchange costs an LDS round trip
+// and the waves do nothing else meanwhile), else one; one when waves share a group, whose sums
+// are then added row by row.
+constexpr int RCH = (TS == 1 && WAVES * kR * NBLK * 512 <= 96 * 1024) ? kR : 1;
+constexpr int SCRATCH_FLOATS = RCH * NBLK * 128;  // per wave
 constexpr int RED_FLOATS = GB * (TS - 1) * NBLK * 128;
 constexpr int GROUP_FLOATS = kR * kS * 64;  // grad_weight values of one group
 constexpr int PUBLISH_FLOATS = WAVES * SCRATCH_FLOATS + RED_FLOATS + (SPIO_PARTIALS ? 0 : GB * GROUP_FLOATS) +
@@ -442,74 +447,130 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
 #else
         float* out = grad_weight;
 #endif
+        if (RCH > 1) {
+            // All filter rows at once: lanes 32-63 leave their halves in the scratch as float4s,
+            // one wave-level sync, lanes 0-31 add them.  LDS operations of a wave execute in order,
+            // so the scratch can be rewritten right after it has been read.
+            spio_float4* half4 = reinterpret_cast<spio_float4*>(scratch);
+            if (lane >= 32) {
 #pragma unroll
-        for (int r = 0; r < kR; ++r) {
-            float total[NBLK][4];
+                for (int r = 0; r < kR; ++r)
 #pragma unroll
-            for (int nb = 0; nb < NBLK; ++nb) {
-                if (lane >= 32) {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) scratch[e * 32 + (lane - 32)] = acc[r + 1][nb][e];
-                }
-                wave_sync();  // lanes 32-63 stored, lanes 0-31 load
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    total[nb][e] = 0.f;
-                    if (lane < 32) total[nb][e] = acc[r][nb][e] + scratch[e * 32 + lane];
-                }
-                wave_sync();  // the scratch is free for the next tap pair
+                    for (int nb = 0; nb < NBLK; ++nb) half4[(r * NBLK + nb) * 32 + (lane - 32)] = acc[r + 1][nb];
             }
-            if (TS > 1) {
-                if (ws > 0 && lane < 32) {
+            wave_sync();  // lanes 32-63 stored, lanes 0-31 load
+            spio_float4 total[kR][NBLK];
 #pragma unroll
-                    for (int nb = 0; nb < NBLK; ++nb)
+            for (int r = 0; r < kR; ++r)
 #pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            red[(((wg * (TS - 1) + ws - 1) * NBLK + nb) * 4 + e) * 32 + lane] = total[nb][e];
+                for (int nb = 0; nb < NBLK; ++nb) {
+                    total[r][nb] = spio_float4{0.f, 0.f, 0.f, 0.f};
+                    if (lane < 32) total[r][nb] = acc[r][nb] + half4[(r * NBLK + nb) * 32 + lane];
                 }
-                block_sync();
-                if (ws == 0 && lane < 32) {
+            wave_sync();  // the halves are read; the scratch becomes the staging area
+#if SPIO_PARTIALS
+            // through the scratch once more, in the partial block's order [r][tap pair][e][32
+            // lanes], so that all 64 lanes store 16 contiguous bytes each
+            if (wave_active) {
+                if (lane < 32) {
 #pragma unroll
-                    for (int w2 = 0; w2 < TS - 1; ++w2)
+                    for (int r = 0; r < kR; ++r)
 #pragma unroll
                         for (int nb = 0; nb < NBLK; ++nb)
 #pragma unroll
-                            for (int e = 0; e < 4; ++e)
-                                total[nb][e] += red[(((wg * (TS - 1) + w2) * NBLK + nb) * 4 + e) * 32 + lane];
-                }
-            }
-#if SPIO_PARTIALS
-            // through the wave's LDS scratch once more so that all 64 lanes store 16 bytes each
-            if (wave_active && ws == 0) {
-                float* stage = scratch;  // NBLK * 128 floats: [tap pair][e][32 lanes]
-                if (lane < 32) {
-#pragma unroll
-                    for (int nb = 0; nb < NBLK; ++nb)
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) stage[(nb * 4 + e) * 32 + lane] = total[nb][e];
+                            for (int e = 0; e < 4; ++e) scratch[((r * NBLK + nb) * 4 + e) * 32 + lane] = total[r][nb][e];
                 }
                 wave_sync();  // lanes 0-31 staged, all lanes load
-                const spio_float4* stage4 = reinterpret_cast<const spio_float4*>(stage);
-                spio_float4* out4 = reinterpret_cast<spio_float4*>(out) + r * NBLK * 32;
+                const spio_float4* stage4 = reinterpret_cast<const spio_float4*>(scratch);
+                spio_float4* out4 = reinterpret_cast<spio_float4*>(out);
 #pragma unroll
-                for (int i = lane; i < NBLK * 32; i += 64) __builtin_nontemporal_store(stage4[i], out4 + i);
-                wave_sync();  // the scratch is free for the next filter row
+                for (int i = lane; i < kR * NBLK * 32; i += 64) __builtin_nontemporal_store(stage4[i], out4 + i);
             }
 #else
-            if (wave_active && ws == 0 && lane < 32) {
+            if (wave_active && lane < 32) {
 #pragma unroll
-                for (int nb = 0; nb < NBLK; ++nb) {
-                    const int s = 2 * nb + sj;
-                    if (s < kS) {
+                for (int r = 0; r < kR; ++r)
 #pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            gstage[(((k4 + e) * kR + r) * kS + s) * 8 + c] = total[nb][e];
+                    for (int nb = 0; nb < NBLK; ++nb) {
+                        const int s = 2 * nb + sj;
+                        if (s < kS) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                gstage[(((k4 + e) * kR + r) * kS + s) * 8 + c] = total[r][nb][e];
+                        }
                     }
-                }
             }
 #endif
-            if (TS > 1) block_sync();  // the scratch is rewritten for the next filter row
-        }
+        } else {
+#pragma unroll
+            for (int r = 0; r < kR; ++r) {
+                float total[NBLK][4];
+    #pragma unroll
+                for (int nb = 0; nb < NBLK; ++nb) {
+                    if (lane >= 32) {
+    #pragma unroll
+                        for (int e = 0; e < 4; ++e) scratch[e * 32 + (lane - 32)] = acc[r + 1][nb][e];
+                    }
+                    wave_sync();  // lanes 32-63 stored, lanes 0-31 load
+    #pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        total[nb][e] = 0.f;
+                        if (lane < 32) total[nb][e] = acc[r][nb][e] + scratch[e * 32 + lane];
+                    }
+                    wave_sync();  // the scratch is free for the next tap pair
+                }
+                if (TS > 1) {
+                    if (ws > 0 && lane < 32) {
+    #pragma unroll
+                        for (int nb = 0; nb < NBLK; ++nb)
+    #pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                red[(((wg * (TS - 1) + ws - 1) * NBLK + nb) * 4 + e) * 32 + lane] = total[nb][e];
+                    }
+                    block_sync();
+                    if (ws == 0 && lane < 32) {
+    #pragma unroll
+                        for (int w2 = 0; w2 < TS - 1; ++w2)
+    #pragma unroll
+                            for (int nb = 0; nb < NBLK; ++nb)
+    #pragma unroll
+                                for (int e = 0; e < 4; ++e)
+                                    total[nb][e] += red[(((wg * (TS - 1) + w2) * NBLK + nb) * 4 + e) * 32 + lane];
+                    }
+                }
+    #if SPIO_PARTIALS
+                // through the wave's LDS scratch once more so that all 64 lanes store 16 bytes each
+                if (wave_active && ws == 0) {
+                    float* stage = scratch;  // NBLK * 128 floats: [tap pair][e][32 lanes]
+                    if (lane < 32) {
+    #pragma unroll
+                        for (int nb = 0; nb < NBLK; ++nb)
+    #pragma unroll
+                            for (int e = 0; e < 4; ++e) stage[(nb * 4 + e) * 32 + lane] = total[nb][e];
+                    }
+                    wave_sync();  // lanes 0-31 staged, all lanes load
+                    const spio_float4* stage4 = reinterpret_cast<const spio_float4*>(stage);
+                    spio_float4* out4 = reinterpret_cast<spio_float4*>(out) + r * NBLK * 32;
+    #pragma unroll
+                    for (int i = lane; i < NBLK * 32; i += 64) __builtin_nontemporal_store(stage4[i], out4 + i);
+                    wave_sync();  // the scratch is free for the next filter row
+                }
+    #else
+                if (wave_active && ws == 0 && lane < 32) {
+    #pragma unroll
+                    for (int nb = 0; nb < NBLK; ++nb) {
+                        const int s = 2 * nb + sj;
+                        if (s < kS) {
+    #pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                gstage[(((k4 + e) * kR + r) * kS + s) * 8 + c] = total[nb][e];
+                        }
+                    }
+                }
+    #endif
+                if (TS > 1) block_sync();  // the scratch is rewritten for the next filter row
+            }
+}
 #if !SPIO_PARTIALS
         // One wave per group adds the group's R*S*64 sums into grad_weight: every atomic
         // instruction covers 64 consecutive floats (two full 128-byte lines), which the memory

@@ -87,7 +87,8 @@ def wgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig) -> Dic
     lds_rings = (nrx * gb * gsx + nrd * (gb * gsd + ((4 - (gb * gsd) % 16) + 16) % 16)) * 16
     # the same LDS block holds the reduction scratch at the end: per-wave row-slot halves, the
     # sums of the other waves of a split group, and (atomic publishing) every group's R*S*64 sums
-    lds_scratch = (gb * ts * (s2 // 2) * 128 + gb * (ts - 1) * (s2 // 2) * 128
+    rch = r if (ts == 1 and gb * ts * r * (s2 // 2) * 512 <= 96 * 1024) else 1  # RCH of the kernel
+    lds_scratch = (gb * ts * rch * (s2 // 2) * 128 + gb * (ts - 1) * (s2 // 2) * 128
                    + (0 if config.two_stage else gb * r * s * 64)
                    + (gb * ts * 8 if params.has_bias else 0)) * 4  # fmt: skip
     g = dict(
