@@ -140,7 +140,11 @@ constexpr int pmod(int a, int m) { return ((a % m) + m) % m; }
 constexpr int RING_UNITS = NRX * XROW_UNITS + NRD * DROW_UNITS;
 constexpr int STREAM_UNITS = RING_UNITS + 2 * OUT_ROW_BYTES / 16;
 constexpr int FILTER_UNITS = GB * 8 * kR * kS;  // filters staged once at the start
-constexpr int SCRATCH_FLOATS = NBLK * 128;      // per wave: row-slot halves
+// Filter rows whose row-slot halves are exchanged through the per-wave scratch in one go: all of
+// them where that fits 96 KB of LDS for the workgroup (every exchange costs an LDS round trip),
+// else one; one when waves share a group, whose sums are then added row by row.
+constexpr int RCH = (TS == 1 && WAVES * kR * NBLK * 512 <= 96 * 1024) ? kR : 1;
+constexpr int SCRATCH_FLOATS = RCH * NBLK * 128;  // per wave: row-slot halves
 constexpr int RED_FLOATS = GB * (TS - 1) * NBLK * 128;
 constexpr int GROUP_FLOATS = kR * kS * 64;
 constexpr int PUBLISH_FLOATS =
@@ -597,54 +601,80 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
         const int k4 = 4 * ((lane >> 4) & 1);
         const int sj = (lane & 15) >> 3;
         const int c = lane & 7;
+        if (RCH > 1) {
+            // all filter rows at once: lanes 32-63 leave their halves in the scratch as float4s, one
+            // wave-level sync, lanes 0-31 add them and stage the sums in grad_weight order
+            spio_float4* half4 = reinterpret_cast<spio_float4*>(scratch);
+            if (lane >= 32) {
 #pragma unroll
-        for (int r = 0; r < kR; ++r) {
-            float total[NBLK][4];
+                for (int r = 0; r < kR; ++r)
 #pragma unroll
-            for (int nb = 0; nb < NBLK; ++nb) {
-                if (lane >= 32) {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) scratch[e * 32 + (lane - 32)] = acc[r + 1][nb][e];
-                }
-                wave_sync();  // lanes 32-63 stored, lanes 0-31 load
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    total[nb][e] = 0.f;
-                    if (lane < 32) total[nb][e] = acc[r][nb][e] + scratch[e * 32 + lane];
-                }
-                wave_sync();  // the scratch is free for the next tap pair
+                    for (int nb = 0; nb < NBLK; ++nb) half4[(r * NBLK + nb) * 32 + (lane - 32)] = acc[r + 1][nb];
             }
-            if (TS > 1) {
-                if (ws > 0 && lane < 32) {
+            wave_sync();  // lanes 32-63 stored, lanes 0-31 load
+            if (wave_active && lane < 32) {
 #pragma unroll
-                    for (int nb = 0; nb < NBLK; ++nb)
+                for (int r = 0; r < kR; ++r)
 #pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            red[(((wg * (TS - 1) + ws - 1) * NBLK + nb) * 4 + e) * 32 + lane] = total[nb][e];
-                }
-                block_sync();
-                if (ws == 0 && lane < 32) {
+                    for (int nb = 0; nb < NBLK; ++nb) {
+                        const spio_float4 total = acc[r][nb] + half4[(r * NBLK + nb) * 32 + lane];
+                        const int s = 2 * nb + sj;
+                        if (s < kS) {
 #pragma unroll
-                    for (int w2 = 0; w2 < TS - 1; ++w2)
-#pragma unroll
-                        for (int nb = 0; nb < NBLK; ++nb)
-#pragma unroll
-                            for (int e = 0; e < 4; ++e)
-                                total[nb][e] += red[(((wg * (TS - 1) + w2) * NBLK + nb) * 4 + e) * 32 + lane];
-                }
+                            for (int e = 0; e < 4; ++e) gstage[(((k4 + e) * kR + r) * kS + s) * 8 + c] = total[e];
+                        }
+                    }
             }
-            if (wave_active && ws == 0 && lane < 32) {
+        } else {
 #pragma unroll
+            for (int r = 0; r < kR; ++r) {
+                float total[NBLK][4];
+    #pragma unroll
                 for (int nb = 0; nb < NBLK; ++nb) {
-                    const int s = 2 * nb + sj;
-                    if (s < kS) {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) gstage[(((k4 + e) * kR + r) * kS + s) * 8 + c] = total[nb][e];
+                    if (lane >= 32) {
+    #pragma unroll
+                        for (int e = 0; e < 4; ++e) scratch[e * 32 + (lane - 32)] = acc[r + 1][nb][e];
+                    }
+                    wave_sync();  // lanes 32-63 stored, lanes 0-31 load
+    #pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        total[nb][e] = 0.f;
+                        if (lane < 32) total[nb][e] = acc[r][nb][e] + scratch[e * 32 + lane];
+                    }
+                    wave_sync();  // the scratch is free for the next tap pair
+                }
+                if (TS > 1) {
+                    if (ws > 0 && lane < 32) {
+    #pragma unroll
+                        for (int nb = 0; nb < NBLK; ++nb)
+    #pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                red[(((wg * (TS - 1) + ws - 1) * NBLK + nb) * 4 + e) * 32 + lane] = total[nb][e];
+                    }
+                    block_sync();
+                    if (ws == 0 && lane < 32) {
+    #pragma unroll
+                        for (int w2 = 0; w2 < TS - 1; ++w2)
+    #pragma unroll
+                            for (int nb = 0; nb < NBLK; ++nb)
+    #pragma unroll
+                                for (int e = 0; e < 4; ++e)
+                                    total[nb][e] += red[(((wg * (TS - 1) + w2) * NBLK + nb) * 4 + e) * 32 + lane];
                     }
                 }
+                if (wave_active && ws == 0 && lane < 32) {
+    #pragma unroll
+                    for (int nb = 0; nb < NBLK; ++nb) {
+                        const int s = 2 * nb + sj;
+                        if (s < kS) {
+    #pragma unroll
+                            for (int e = 0; e < 4; ++e) gstage[(((k4 + e) * kR + r) * kS + s) * 8 + c] = total[nb][e];
+                        }
+                    }
+                }
+                if (TS > 1) block_sync();  // the scratch is rewritten for the next filter row
             }
-            if (TS > 1) block_sync();  // the scratch is rewritten for the next filter row
-        }
+}
         if (wave_active && ws == 0) {
             float* gout = grad_weight + (long long)gglob * GROUP_FLOATS;
             wave_sync();  // lanes 0-31 staged the sums, all lanes read them

@@ -96,7 +96,8 @@ def bgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig) -> Dic
     out_row_bytes = 16 * wt * (gb * 16 + 16)
     stream_bytes = ring_units * 16 + 2 * out_row_bytes
     filter_bytes = gb * 8 * r * s * 16
-    publish_bytes = (gb * ts * nblk * 128 + gb * (ts - 1) * nblk * 128 + gb * r * s * 64
+    rch = r if (ts == 1 and gb * ts * r * nblk * 512 <= 96 * 1024) else 1  # RCH of the kernel
+    publish_bytes = (gb * ts * rch * nblk * 128 + gb * (ts - 1) * nblk * 128 + gb * r * s * 64
                      + (gb * ts * 8 if params.has_bias else 0)) * 4  # fmt: skip
     lptx = divup(f * gb, threads)
     lptd = divup(nb * params.q * gb, threads)
