@@ -1,8 +1,9 @@
 """Every shape of the reference's kernel-test lists (spio/src_tests/Conv2dGw8Params.dat and the
 parameter grid of tests/test_conv2d_gw8.py: 270 shapes here), every kernel family, against the
-CPU oracle: by default the first (best-ranked) MFMA configuration of every kernel for every shape
-and one random other configuration for every third shape (a few minutes on one MI355X);
-SPIO_EXHAUSTIVE=1 takes five random configurations per kernel instead (about 15 minutes).
+CPU oracle: by default the first (best-ranked) configuration of every MFMA kernel (row-streaming
+and, where the shape has one, whole-image) for every shape and one random other configuration for
+every third shape (a few minutes on one MI355X); SPIO_EXHAUSTIVE=1 takes five configurations per
+kernel family instead (about 15 minutes).
 """
 
 import os
@@ -31,10 +32,14 @@ CONFIGS_PER_KERNEL = 5
 
 
 def _pick(factory, params, attr, rng, second=True, **kw):
-    configs = [c for c in factory.configs(params, attr, **kw) if getattr(c, "variant", "mfma") == "mfma"]
+    every = list(factory.configs(params, attr, **kw))
+    rows = [c for c in every if getattr(c, "variant", "mfma") == "mfma"]    # row-streaming kernels
+    image = [c for c in every if getattr(c, "variant", "mfma") == "image"]  # whole-image kernel
+    first = rows[:1] + image[:1]
+    rest = rows[1:] + image[1:]
     if FULL:
-        return rng.sample(configs, min(CONFIGS_PER_KERNEL, len(configs)))
-    return configs[:1] + (rng.sample(configs[1:], 1) if second and len(configs) > 1 else [])
+        return first + rng.sample(rest, min(CONFIGS_PER_KERNEL - len(first), len(rest)))
+    return first + (rng.sample(rest, 1) if second and rest else [])
 
 
 @pytest.mark.parametrize("chunk", range((len(SHAPES) + CHUNK - 1) // CHUNK))
