@@ -215,8 +215,13 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
             b = (k / CH) * (8 * CH) + x8 * CH + k % CH;
         }
     }
-    const int pb = b % PBLKS;
-    const int cb = (b / PBLKS) % GBLKS;
+    // Tile order: row blocks fastest, so that neighbours in a run share halo rows.  Where a
+    // workgroup covers only part of a pixel's 128-byte lines (GB * 16 bytes per pixel), the channel
+    // blocks that share those lines go fastest instead: dealt to different XCDs, every one of
+    // them would fetch the whole lines from memory (measured: twice the algorithmic reads).
+    constexpr bool kSplitLines = GBLKS > 1 && (GB * 16) % 128 != 0;
+    const int pb = kSplitLines ? (b / GBLKS) % PBLKS : b % PBLKS;
+    const int cb = kSplitLines ? b % GBLKS : (b / PBLKS) % GBLKS;
     const int nbk = b / (PBLKS * GBLKS);
     const int p0 = pb * BH;
     const int bh_eff = imin(BH, kP - p0);  // rows this block owns
