@@ -33,7 +33,8 @@ MAX_LOADS_PER_THREAD = 8
 MAX_ACCUMULATORS = 16
 MAX_CONFIGS = 36
 DEVICE_LDS_BYTES = 160 * 1024
-MAX_IMAGE_CONFIGS = 8  # whole-image configurations that enter the sweep
+MAX_IMAGE_CONFIGS = 10  # whole-image configurations that enter the sweep
+MOVER_WAVES = 4  # data-mover waves of the whole-image kernel where it has any: one per SIMD
 PREFETCH_CHOICES = (2, 4, 8, 12, 16)
 MAX_GEOMETRIES = 24  # tile geometries that enter the sweep; the best few also try the other cache/XCD policies
 
@@ -62,6 +63,9 @@ class Conv2dGw8Config:
             output, prefetch = 1 one of each, which lets two workgroups share a CU; block_p and
             the cache/XCD policies do not apply) or "direct" (one thread per output
             pixel-group; any shape).
+        movers: whole-image kernel only: extra waves that move the image blocks between global
+            memory and LDS for the whole workgroup while the other waves only multiply (0: every
+            wave does both).
     """
 
     groups: int = 8
@@ -74,6 +78,7 @@ class Conv2dGw8Config:
     halo_cached: int = 1
     xcd_chunk: int = 4
     block_n_iters: int = 1
+    movers: int = 0
 
 
 def direction_geometry(params: Conv2dGw8Params, igrad: bool) -> Dict[str, int]:
@@ -126,23 +131,31 @@ def image_geometry(params: Conv2dGw8Params, config: Conv2dGw8Config, igrad: bool
     wt = divup(f - s + 1, 16)
     fp = 16 * wt + 4 * kb - 1
     gs = fp + ((9 - fp % 16) + 16) % 16
-    threads = 64 * gb * ts
+    threads = 64 * (gb * ts + config.movers)
+    mthreads = 64 * config.movers if config.movers else threads  # threads that move image blocks
     nbuf = 2 if config.prefetch >= 2 else 1  # prefetch = 1: single buffers (SPIO_DB = 0)
     in_units = d["SH"] * gb * gs
     out_bytes = d["DH"] * 16 * wt * (gb * 16 + 16)
     # input buffers, dump cells, output buffers (which first hold the groups' filters)
     lds = (nbuf * in_units + 32) * 16 + max(nbuf * out_bytes, gb * 8 * r * s * 16)
-    lpt = divup(d["SH"] * nb * d["SW"] * gb, threads)
-    spt = divup(d["DH"] * nb * d["DW"] * gb, threads)
-    wlpt = divup(gb * 8 * r * s, threads)
+    lpt = divup(d["SH"] * nb * d["SW"] * gb, mthreads)
+    spt = divup(d["DH"] * nb * d["DW"] * gb, mthreads)
+    wlpt = divup(gb * 8 * r * s, 64 * gb * ts)  # the multiplying waves fetch the filters
     apw = max(nacc // max(ts, 1), 1)
+    # registers per lane.  Multiplying: filter fragments, accumulators, two sets of source
+    # fragments; moving: two blocks in flight and their LDS addresses; both: the filter share on
+    # its way to LDS and the rest.  Without mover waves every wave holds both sets.
+    multiplying = 4 * ns * kb + 4 * wt * apw + 8 * wt * kb
+    moving = 8 * lpt + lpt + spt
+    if config.movers:
+        registers = max(multiplying + 4 * wlpt, moving) + 14
+    else:
+        registers = multiplying + 4 * max(2 * lpt, lpt + wlpt) + lpt + spt + 14
     d.update(
         NS=ns, NACC=nacc, APW=apw, KB=kb, WPI=wpi, F=f, WT=wt, GS=gs, THREADS=threads,
-        LDS_BYTES=lds, LPT=lpt, SPT=spt, STEPS=d["DH"] + r - 1,
+        MTHREADS=mthreads, LDS_BYTES=lds, LPT=lpt, SPT=spt, STEPS=d["DH"] + r - 1,
         GBLKS=divup(params.groups, gb), NBLKS=divup(params.n, nb),
-        # filter fragments, accumulators, source fragments, block in flight, addressing, the rest
-        REGISTERS=4 * ns * kb + 4 * wt * apw + 8 * wt * kb + 4 * max(2 * lpt, lpt + wlpt) + 2 * (lpt + spt) + 14,
-        NBUF=nbuf,
+        REGISTERS=registers, NBUF=nbuf,
     )  # fmt: skip
     d["WGBLKS"] = divup(d["NBLKS"], iters)
     d["NUM_BLOCKS"] = d["GBLKS"] * d["WGBLKS"]
@@ -151,9 +164,14 @@ def image_geometry(params: Conv2dGw8Params, config: Conv2dGw8Config, igrad: bool
 
 def _image_config_is_legal(params, config, igrad) -> bool:
     g = image_geometry(params, config, igrad)
-    waves = config.groups * config.split
+    waves = config.groups * config.split + config.movers
+    # registers per lane that leave room for the workgroup's waves on a SIMD (512 in all)
+    budget = {1: 232, 2: 232, 3: 160, 4: 128}.get(divup(waves, 4), 0)
     return (
         waves <= MAX_WAVES
+        and config.movers >= 0
+        and (config.movers == 0 or (config.prefetch >= 2 and g["MTHREADS"] % config.groups == 0))
+        and g["THREADS"] % config.groups == 0
         and config.split >= 1
         and g["NACC"] % config.split == 0
         and config.block_n <= max(params.n, 1)
@@ -162,8 +180,7 @@ def _image_config_is_legal(params, config, igrad) -> bool:
         and g["LPT"] <= MAX_LOADS_PER_THREAD
         and g["SPT"] <= MAX_LOADS_PER_THREAD
         and g["STEPS"] <= MAX_UNROLLED_STEPS
-        # registers per lane: 128 where a SIMD must hold four waves of the workgroup, else 256
-        and g["REGISTERS"] <= (128 if waves > 8 else 232)
+        and g["REGISTERS"] <= budget
         and config.block_n * params.c * max(params.h * params.w, params.p * params.q) * 2 < 2**31
     )
 
@@ -184,8 +201,11 @@ def _image_score(params, config, igrad, num_cus: int) -> float:
     setup = 1.0 + 2.0 / config.block_n_iters
     split = 1.0 + 0.05 * (config.split - 1)
     single = 1.0 if config.prefetch >= 2 else 1.03
+    # mover waves pay where moving a block takes longer than multiplying it (measured: 3x3 on
+    # 14x14 0.73x, 7x7 on 14x14 1.05x)
+    movers = 1.0 if not config.movers else (0.9 if params.r * params.s < 25 else 1.05)
     ragged = g["WGBLKS"] * config.block_n_iters * config.block_n / params.n
-    return quant * ragged * split_line * setup * split * single / (tile_eff * group_eff)
+    return quant * ragged * split_line * setup * split * single * movers / (tile_eff * group_eff)
 
 
 def _image_configs(params: Conv2dGw8Params, igrad: bool, num_cus: int) -> List[Conv2dGw8Config]:
@@ -196,10 +216,11 @@ def _image_configs(params: Conv2dGw8Params, igrad: bool, num_cus: int) -> List[C
         for nb in (1, 2, 4, 8):
             for ts in (1, 2, 4):
                 for iters in (1, 2, 4, 8, 16):
-                    for buffers in (2, 1):
+                    for buffers, movers in ((2, 0), (1, 0), (2, MOVER_WAVES)):
                         cfg = Conv2dGw8Config(groups=gb, block_p=direction_geometry(params, igrad)["DH"],
                                               block_n=nb, split=ts, prefetch=buffers, variant="image",
-                                              halo_cached=0, xcd_chunk=0, block_n_iters=iters)  # fmt: skip
+                                              halo_cached=0, xcd_chunk=0, block_n_iters=iters,
+                                              movers=movers)  # fmt: skip
                         if nb * iters > max(params.n, 1) and iters > 1:
                             continue
                         if _image_config_is_legal(params, cfg, igrad):
@@ -326,7 +347,7 @@ def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8Config, _device_a
         defines.update(
             SPIO_GB=config.groups, SPIO_NB=config.block_n, SPIO_TS=config.split,
             SPIO_ITERS=config.block_n_iters, SPIO_NT=config.nontemporal,
-            SPIO_DB=int(config.prefetch >= 2),
+            SPIO_DB=int(config.prefetch >= 2), SPIO_MV=config.movers,
         )  # fmt: skip
         return KernelSpec(
             defines, LaunchParams(grid=g["NUM_BLOCKS"], block=g["THREADS"]), IMAGE_SOURCE, notes=g

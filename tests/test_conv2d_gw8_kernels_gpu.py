@@ -117,9 +117,14 @@ def test_fprop_explicit_configs():
                     configs=[Conv2dGw8Config(groups=8, block_p=8, block_n=1)])  # fmt: skip
 
 
-def _image(groups, block_n, split, iters, buffers=2):
+def _image(groups, block_n, split, iters, buffers=2, movers=0):
     return Conv2dGw8Config(groups=groups, block_p=0, block_n=block_n, split=split, prefetch=buffers,
-                           variant="image", block_n_iters=iters, halo_cached=0, xcd_chunk=0)  # fmt: skip
+                           variant="image", block_n_iters=iters, halo_cached=0, xcd_chunk=0,
+                           movers=movers)  # fmt: skip
+
+
+def _movers(groups, block_n, split, iters, movers=4):
+    return _image(groups, block_n, split, iters, 2, movers)
 
 
 IMAGE_CASES = [
@@ -127,17 +132,21 @@ IMAGE_CASES = [
     # a batch that does not fill the last workgroup's blocks
     (Conv2dGw8Params(n=7, c=64, h=14, w=14, r=7, s=7, padding=3),
      [_image(8, 1, 1, 1), _image(8, 1, 1, 5), _image(4, 1, 4, 2), _image(4, 1, 2, 3, 1), _image(4, 1, 2, 16),
-      _image(8, 1, 1, 2, 1), _image(4, 2, 2, 3, 1)]),
+      _image(8, 1, 1, 2, 1), _image(4, 2, 2, 3, 1),
+      # data-mover waves: 1..5 blocks per workgroup, split accumulators, two mover waves
+      _movers(8, 1, 1, 1), _movers(8, 1, 1, 4), _movers(4, 1, 2, 5), _movers(4, 1, 1, 2, movers=2), _movers(2, 2, 2, 3)]),
     # 3x3 with a bias, images side by side, a group count that leaves idle waves (5 groups, 4 per block)
     (Conv2dGw8Params(n=9, c=40, h=14, w=14, has_bias=True),
-     [_image(4, 2, 1, 2), _image(4, 1, 2, 1, 1), _image(5, 1, 1, 4), _image(2, 4, 2, 1), _image(5, 2, 1, 3, 1)]),
+     [_image(4, 2, 1, 2), _image(4, 1, 2, 1, 1), _image(5, 1, 1, 4), _image(2, 4, 2, 1), _image(5, 2, 1, 3, 1),
+      _movers(4, 2, 1, 2), _movers(5, 1, 1, 4, movers=5), _movers(2, 4, 2, 1)]),
     # 7x7 images
-    (Conv2dGw8Params(n=12, c=64, h=7, w=7, has_bias=True), [_image(8, 2, 1, 2), _image(8, 2, 2, 1), _image(4, 4, 1, 3), _image(8, 4, 1, 3, 1)]),
+    (Conv2dGw8Params(n=12, c=64, h=7, w=7, has_bias=True), [_image(8, 2, 1, 2), _image(8, 2, 2, 1), _image(4, 4, 1, 3), _image(8, 4, 1, 3, 1),
+      _movers(8, 2, 1, 2), _movers(4, 4, 1, 3)]),
     # 5x5 (three accumulators: splits 1 and 3), non-square image
-    (Conv2dGw8Params(n=5, c=32, h=9, w=12, r=5, s=5, padding=2, has_bias=True), [_image(4, 1, 3, 2), _image(4, 2, 1, 2, 1)]),
+    (Conv2dGw8Params(n=5, c=32, h=9, w=12, r=5, s=5, padding=2, has_bias=True), [_image(4, 1, 3, 2), _image(4, 2, 1, 2, 1), _movers(4, 1, 3, 2)]),
     # asymmetric filter and padding, output larger than the input (the data gradient then crops)
-    (Conv2dGw8Params(n=3, c=16, h=6, w=8, r=3, s=3, padding=2), [_image(2, 1, 1, 2), _image(2, 2, 2, 1), _image(2, 1, 1, 3, 1)]),
-    (Conv2dGw8Params(n=4, c=16, h=10, w=6, r=4, s=1, padding=(2, 0), has_bias=True), [_image(2, 2, 2, 2)]),
+    (Conv2dGw8Params(n=3, c=16, h=6, w=8, r=3, s=3, padding=2), [_image(2, 1, 1, 2), _image(2, 2, 2, 1), _image(2, 1, 1, 3, 1), _movers(2, 1, 1, 3)]),
+    (Conv2dGw8Params(n=4, c=16, h=10, w=6, r=4, s=1, padding=(2, 0), has_bias=True), [_image(2, 2, 2, 2), _movers(2, 2, 2, 2)]),
     (Conv2dGw8Params(n=2, c=16, h=8, w=8, r=3, s=3, padding=0), [_image(2, 1, 1, 2)]),
 ]
 
