@@ -53,11 +53,23 @@ union Pack {
     ln_half8 h;
 };
 
-// Sum over the LPP lanes of a pixel; every lane ends up with the total.
+// Sum over the LPP lanes of a pixel; every lane ends up with the total.  Inside a row of 16
+// lanes the partner's value comes through the data-parallel-primitive operand path (swap inside
+// pairs, swap the pairs of a quad, mirror the halves of 8, mirror the row); beyond a row through
+// the LDS crossbar.
+template <int CTRL>
+__device__ inline float dpp_add(float v) {
+    const int other = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false);
+    return v + __builtin_bit_cast(float, other);
+}
 __device__ inline float pixel_sum(float v) {
+    if (LPP >= 2) v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+    if (LPP >= 4) v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+    if (LPP >= 8) v = dpp_add<0x141>(v);  // row_half_mirror: lane i of 8 <-> lane 7-i
+    if (LPP >= 16) v = dpp_add<0x140>(v); // row_mirror: lane i of 16 <-> lane 15-i
     const int lane = (int)__builtin_amdgcn_workitem_id_x() & 63;
 #pragma unroll
-    for (int m = 1; m < LPP; m <<= 1) {
+    for (int m = 16; m < LPP; m <<= 1) {
         const int other = __builtin_amdgcn_ds_bpermute(((lane ^ m) << 2), __builtin_bit_cast(int, v));
         v += __builtin_bit_cast(float, other);
     }

@@ -66,11 +66,15 @@ class LayerNorm2dParams:
 
 @dataclass(frozen=True)
 class LayerNorm2dConfig:
-    """threads per workgroup, pixel groups in flight per lane, workgroups per compute unit."""
+    """threads per workgroup, pixel groups in flight per lane, workgroups per compute unit, and
+    the lanes that share a pixel (0: the smallest power of two that gives every 16-byte unit of a
+    pixel its own lane; a smaller power of two gives each lane several units, which keeps all
+    lanes busy when C/8 is not a power of two: 96 channels = 12 units = 4 lanes x 3 units)."""
 
     threads: int = 256
     unroll: int = 4
     groups_per_cu: int = 8
+    lanes: int = 0
 
 
 def lanes_per_pixel(c: int) -> int:
@@ -81,22 +85,45 @@ def lanes_per_pixel(c: int) -> int:
     return lpp
 
 
+def _lane_choices(c: int) -> List[int]:
+    """Lanes per pixel worth trying: the default, and where that leaves lanes idle the largest
+    power of two that divides the units of a pixel (at most 4 units per lane)."""
+    units = c // 8
+    full = lanes_per_pixel(c)
+    out = [0]
+    if full != units:
+        exact = units & -units  # largest power of two dividing units
+        if exact < full and divup(units, exact) <= 4:
+            out.append(exact)
+    return out
+
+
 def _get_configs(params: LayerNorm2dParams, _device_attr=None) -> List[LayerNorm2dConfig]:
-    upl = divup(params.c // 8, lanes_per_pixel(params.c))
+    per_lanes = []
+    for lanes in _lane_choices(params.c):
+        upl = divup(params.c // 8, lanes or lanes_per_pixel(params.c))
+        mine = []
+        for threads in (256, 512):
+            for unroll in (8, 4, 2, 1):  # as many loads in flight as the registers hold
+                if unroll * upl > 8:
+                    continue
+                for per_cu in (8, 16, 4):
+                    mine.append(LayerNorm2dConfig(threads, unroll, per_cu, lanes))
+        per_lanes.append(mine)
+    # the lane choices alternate, busy lanes first, so that a sweep cut short has seen both
     out = []
-    for threads in (256, 512):
-        for unroll in (4, 2, 8):
-            if unroll * upl > 8:
-                continue
-            for per_cu in (8, 4, 16):
-                out.append(LayerNorm2dConfig(threads, unroll, per_cu))
+    for i in range(max(len(m) for m in per_lanes)):
+        for mine in reversed(per_lanes):
+            if i < len(mine):
+                out.append(mine[i])
     return out or [LayerNorm2dConfig(256, 1, 8)]
 
 
 def _get_kernel_spec(params: LayerNorm2dParams, config: LayerNorm2dConfig, device_attr=None) -> KernelSpec:
     params.validate()
     cus = getattr(device_attr, "multiprocessor_count", 256) or 256
-    lpp = lanes_per_pixel(params.c)
+    lpp = config.lanes or lanes_per_pixel(params.c)
+    assert lpp & (lpp - 1) == 0 and lpp <= 64 and divup(params.c // 8, lpp) <= 4, f"illegal configuration {config}"
     pass_pixels = (64 // lpp) * (config.threads // 64) * config.unroll
     grid = max(1, min(divup(params.pixels, pass_pixels), cus * config.groups_per_cu))
     defines = {
