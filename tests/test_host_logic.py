@@ -52,6 +52,14 @@ def test_every_shape_has_legal_configs(igrad):
                 assert spec.launch_params.grid[0] == g["NUM_BLOCKS"] == g["GBLKS"] * g["WGBLKS"]
                 assert spec.launch_params.block[0] == g["THREADS"]
                 assert g["WGBLKS"] * cfg.block_n_iters * cfg.block_n >= params.n
+                # data-mover waves come on top of the multiplying waves, need the second pair of
+                # buffers, and a moving thread stays with one group
+                assert g["THREADS"] == 64 * (cfg.groups * cfg.split + cfg.movers)
+                assert g["MTHREADS"] == (64 * cfg.movers if cfg.movers else g["THREADS"])
+                assert g["MTHREADS"] % cfg.groups == 0
+                assert spec.defines["SPIO_MV"] == cfg.movers
+                if cfg.movers:
+                    assert cfg.prefetch >= 2 and spec.defines["SPIO_DB"] == 1
                 continue
             g = mfma_geometry(params, cfg, igrad)
             assert g["THREADS"] <= 1024 and g["LDS_BYTES"] <= MAX_LDS_BYTES
@@ -218,3 +226,43 @@ def test_tuner_record_store(tmp_path, monkeypatch):
     assert Tuner().lookup(ATTR, "k__x")["us"] == 12.5
     assert device_key(ATTR) == "gfx950_256cu"
     assert json.load(open(tmp_path / "db.json"))["k__x"]["config"] == {"groups": 8}
+
+
+def test_small_image_shapes_offer_mover_wave_configurations():
+    """The whole-image kernel is offered with and without data-mover waves for the small-image
+    shapes; for 3x3 filters both are among the first candidates (a sweep cut short sees both)."""
+    for shape in ("128n_384c_14h_14w_1py_1px_3r_3s_b", "256n_256c_14h_14w_3py_3px_7r_7s_nb"):
+        params = Conv2dGw8Params.decode(shape)
+        configs = conv2d_gw8_kernel_factory.configs(params, ATTR)
+        image = [c for c in configs if c.variant == "image"]
+        assert any(c.movers for c in image) and any(not c.movers for c in image)
+        if params.r == 3:  # where moving a block takes longer than multiplying it
+            assert {bool(c.movers) for c in configs[:4] if c.variant == "image"} == {False, True}
+    # illegal: mover waves with single buffers, or more waves than a workgroup holds
+    params = Conv2dGw8Params.decode("128n_384c_14h_14w_1py_1px_3r_3s_b")
+    for bad in (Conv2dGw8Config(groups=8, block_p=14, variant="image", prefetch=1, movers=4, block_n_iters=2),
+                Conv2dGw8Config(groups=8, block_p=14, variant="image", prefetch=2, movers=12, block_n_iters=2)):
+        with pytest.raises(AssertionError):
+            conv2d_gw8_kernel_factory.get_kernel_spec(params, bad, ATTR)
+
+
+def test_layernorm_lane_choices():
+    """Lanes per pixel: one unit per lane by default; where C/8 is not a power of two also the
+    largest power of two dividing it, both among the first candidates."""
+    from spio_amd.kernels import LayerNorm2dParams, layernorm_2d_kernel_factory
+
+    expected = {96: 4, 192: 8, 384: 16, 768: 32, 64: None, 40: None, 2048: None}
+    for c, exact in expected.items():
+        params = LayerNorm2dParams(n=2, c=c, h=3, w=5)
+        configs = layernorm_2d_kernel_factory.configs(params, ATTR)
+        assert len(set(configs)) == len(configs)
+        lanes = {cfg.lanes for cfg in configs}
+        assert lanes == ({0, exact} if exact else {0})
+        if exact:
+            assert {cfg.lanes for cfg in configs[:2]} == {0, exact}
+        for cfg in configs:
+            spec = layernorm_2d_kernel_factory.get_kernel_spec(params, cfg, ATTR)
+            lpp = spec.defines["SPIO_LN_LPP"]
+            upl = -(-(c // 8) // lpp)
+            assert lpp & (lpp - 1) == 0 and lpp * upl >= c // 8 and cfg.unroll * upl <= 8
+
