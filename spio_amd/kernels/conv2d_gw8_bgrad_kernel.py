@@ -159,11 +159,23 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None) -> List[Conv2dGw8Bgr
     # whether whole images or row blocks win depends on the shape in ways the score does not
     # capture (contiguity of the channel block, halo re-reads, workgroups per compute unit).
     row_choices = [0] + sorted({bh for bh in (7, 14, 28) if bh < params.p}, reverse=True)
+    # images side by side: powers of two, and for rows shorter than a 32-pixel chunk of the weight
+    # gradient's contraction the counts that fill the chunks clearly better (as in the
+    # weight-gradient kernel's configuration space)
+    wpi = params.q + params.s - 1
+
+    def chunk_fill(nb):
+        return nb * params.q / (32.0 * divup((nb - 1) * wpi + params.q, 32))
+
+    image_counts = [1, 2, 4, 8]
+    if wpi < 32:
+        best = max(chunk_fill(nb) for nb in image_counts)
+        image_counts += [nb for nb in (3, 5, 6, 7) if chunk_fill(nb) > best + 0.05]
     configs = []
     for bh in row_choices:
         geometries = []
         for gb in group_choices:
-            for nb in (1, 2, 4, 8):
+            for nb in image_counts:
                 for iters in (1, 2, 4):
                     for ts in (1, 2):
                         cfg = Conv2dGw8BgradConfig(groups=gb, block_h=bh, block_n=nb, block_n_iters=iters,

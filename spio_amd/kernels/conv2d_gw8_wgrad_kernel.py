@@ -150,11 +150,24 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None) -> List[Conv2dGw8Wgr
     G = params.groups
     group_choices = sorted({g for g in (4, 8, 16, G) if g <= min(G, MAX_WAVES)}) or [min(G, MAX_WAVES)]
     row_choices = sorted({bh for bh in (4, 7, 8, 14, 16, 28, 32, 56, params.p) if bh <= params.p})
+    # Images side by side.  The contraction runs over 32-pixel chunks of the flattened row, so
+    # where a padded image row is shorter than a chunk the count decides how full the chunks
+    # are: besides the powers of two, the counts that fill them clearly better (7x7 images with
+    # one halo column each side: 8 images fill 56 of 96 pixels, 7 images 49 of 64).
+    wpi = params.q + params.s - 1
+
+    def chunk_fill(nb):
+        return nb * params.q / (32.0 * divup((nb - 1) * wpi + params.q, 32))
+
+    image_counts = [1, 2, 4, 8]
+    if wpi < 32:
+        best = max(chunk_fill(nb) for nb in image_counts)
+        image_counts += [nb for nb in (3, 5, 6, 7) if chunk_fill(nb) > best + 0.05]
     # Rank the tile geometries first and keep the best few; each of them is then tried with the
     # pipeline variants (prefetch distance, rows per step), which the score cannot tell apart.
     geometries = []
     for gb in group_choices:
-        for nb in (1, 2, 4, 8):
+        for nb in image_counts:
             for iters in (1, 2, 4, 8):
                 for bh in row_choices:
                     for two_stage in (0, 1):
