@@ -98,6 +98,21 @@ def test_bgrad_explicit_configs():
                                    Conv2dGw8BgradConfig(groups=2, block_h=4, block_n=1, block_n_iters=1, prefetch=2, split=1)])  # fmt: skip
 
 
+def test_odd_image_counts_on_small_images():
+    """7x7 images: 3 and 7 images side by side fill the 32-pixel chunks of the weight gradient's
+    contraction better than powers of two; a batch that leaves the last block ragged."""
+    from spio_amd.kernels import Conv2dGw8WgradConfig
+
+    params = Conv2dGw8Params(n=17, c=64, h=7, w=7, padding=1, has_bias=True)
+    run_grad_kernel_test(conv2d_gw8_wgrad_kernel_factory, params,
+                         configs=[Conv2dGw8WgradConfig(groups=4, block_h=7, block_n=7, block_n_iters=1, prefetch=4),
+                                  Conv2dGw8WgradConfig(groups=8, block_h=7, block_n=7, block_n_iters=2, prefetch=2, rows=2),
+                                  Conv2dGw8WgradConfig(groups=4, block_h=4, block_n=3, block_n_iters=2, prefetch=2, two_stage=1)])  # fmt: skip
+    run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params,
+                          configs=[Conv2dGw8BgradConfig(groups=8, block_h=0, block_n=7, block_n_iters=1, prefetch=2, split=1),
+                                   Conv2dGw8BgradConfig(groups=4, block_h=0, block_n=3, block_n_iters=2, prefetch=4, split=1)])  # fmt: skip
+
+
 def test_bgrad_is_not_offered_when_the_image_size_changes():
     assert not bgrad_is_supported(Conv2dGw8Params(n=1, c=8, h=8, w=8, padding=0))
     assert not bgrad_is_supported(Conv2dGw8Params(n=1, c=8, h=8, w=8, r=4, s=1, padding=(2, 0)))
