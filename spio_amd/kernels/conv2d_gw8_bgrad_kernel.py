@@ -154,7 +154,10 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None) -> List[Conv2dGw8Bgr
     """Legal configurations, most promising first; empty when the shape is not supported."""
     num_cus = getattr(device_attr, "multiprocessor_count", 256) or 256
     G = params.groups
-    group_choices = sorted({g for g in (4, 8, 16, G) if g <= min(G, MAX_WAVES)}) or [min(G, MAX_WAVES)]
+    # powers of two, the whole pixel, and half a pixel where the group count is not a power of two
+    # (96 channels: 12 groups = 2 x 6)
+    group_choices = sorted({g for g in (4, 8, 16, G, G // 2 if G % 2 == 0 and G & (G - 1) else G)
+                            if 0 < g <= min(G, MAX_WAVES)}) or [min(G, MAX_WAVES)]
     # Rank the geometries of every row-block height separately and keep the best few of each:
     # whether whole images or row blocks win depends on the shape in ways the score does not
     # capture (contiguity of the channel block, halo re-reads, workgroups per compute unit).

@@ -148,7 +148,10 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None) -> List[Conv2dGw8Wgr
     """Legal configurations, most promising first; a direct-kernel configuration closes the list."""
     num_cus = getattr(device_attr, "multiprocessor_count", 256) or 256
     G = params.groups
-    group_choices = sorted({g for g in (4, 8, 16, G) if g <= min(G, MAX_WAVES)}) or [min(G, MAX_WAVES)]
+    # powers of two, the whole pixel, and half a pixel where the group count is not a power of two
+    # (96 channels: 12 groups = 2 x 6)
+    group_choices = sorted({g for g in (4, 8, 16, G, G // 2 if G % 2 == 0 and G & (G - 1) else G)
+                            if 0 < g <= min(G, MAX_WAVES)}) or [min(G, MAX_WAVES)]
     row_choices = sorted({bh for bh in (4, 7, 8, 14, 16, 28, 32, 56, params.p) if bh <= params.p})
     # Images side by side.  The contraction runs over 32-pixel chunks of the flattened row, so
     # where a padded image row is shorter than a chunk the count decides how full the chunks
