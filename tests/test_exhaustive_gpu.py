@@ -1,7 +1,7 @@
 """Every shape of the reference's kernel-test lists (spio/src_tests/Conv2dGw8Params.dat and the
 parameter grid of tests/test_conv2d_gw8.py: 270 shapes here), every kernel family, against the
 CPU oracle: by default the first (best-ranked) configuration of every MFMA kernel (row-streaming
-and, where the shape has one, whole-image) for every shape and one random other configuration for
+and, where the shape has one, whole-image with and without mover waves) for every shape and one random other configuration for
 every third shape (a few minutes on one MI355X); SPIO_EXHAUSTIVE=1 takes five configurations per
 kernel family instead (about 15 minutes).
 """
@@ -35,8 +35,10 @@ def _pick(factory, params, attr, rng, second=True, **kw):
     every = list(factory.configs(params, attr, **kw))
     rows = [c for c in every if getattr(c, "variant", "mfma") == "mfma"]    # row-streaming kernels
     image = [c for c in every if getattr(c, "variant", "mfma") == "image"]  # whole-image kernel
-    first = rows[:1] + image[:1]
-    rest = rows[1:] + image[1:]
+    movers = [c for c in image if getattr(c, "movers", 0)]                  # ... with data-mover waves
+    plain = [c for c in image if not getattr(c, "movers", 0)]
+    first = rows[:1] + plain[:1] + movers[:1]
+    rest = [c for c in rows + image if c not in first]
     if FULL:
         return first + rng.sample(rest, min(CONFIGS_PER_KERNEL - len(first), len(rest)))
     return first + (rng.sample(rest, 1) if second and rest else [])
