@@ -2,6 +2,7 @@
 
     python -m spio_amd.tune --shapes bench            # the benchmark shapes
     python -m spio_amd.tune 128n_64c_56h_56w_1py_1px_3r_3s_nb [...]
+    python -m spio_amd.tune 128n_96c_56h_56w_1em06eps_wb      # a LayerNorm2d shape
     python -m spio_amd.tune --shapes bench --package  # write into the package's own records
 
 Records land in the user cache (or SPIO_TUNE_DB) unless --package is given; later processes
@@ -27,6 +28,11 @@ NETWORK_SHAPES = [
     "128n_192c_28h_28w_1py_1px_3r_3s_b",
     "128n_384c_14h_14w_1py_1px_3r_3s_b",
     "128n_768c_7h_7w_1py_1px_3r_3s_b",
+    # the channel LayerNorms of the same network (LayerNorm2dParams.encode() form)
+    "128n_96c_56h_56w_1em06eps_wb",
+    "128n_192c_28h_28w_1em06eps_wb",
+    "128n_384c_14h_14w_1em06eps_wb",
+    "128n_768c_7h_7w_1em06eps_wb",
 ]
 
 
@@ -196,9 +202,11 @@ def main(argv=None):
     from .hip import get_device_attributes
     from .kernels import (
         Conv2dGw8Params,
+        LayerNorm2dParams,
         conv2d_gw8_bgrad_kernel_factory,
         conv2d_gw8_kernel_factory,
         conv2d_gw8_wgrad_kernel_factory,
+        layernorm_2d_kernel_factory,
     )
     from .kernels.tuner import _PACKAGE_RECORDS, device_key, tuner
 
@@ -229,6 +237,15 @@ def main(argv=None):
         if shape in seen:
             continue
         seen.add(shape)
+        if "eps_" in shape:  # a LayerNorm2d shape: one kernel family, no directions
+            params = LayerNorm2dParams.decode(shape)
+            kernel = tuner.sweep(layernorm_2d_kernel_factory, params, 0, attr, warmup=3, iters=args.iters,
+                                 record_path=path)  # fmt: skip
+            best = min(r["us"] for r in tuner.last_sweep if "us" in r)
+            print(f"lnorm {shape}: {best:8.1f} us  {kernel.config}", flush=True)
+            kernel.unload()
+            torch.cuda.empty_cache()
+            continue
         params = Conv2dGw8Params.decode(shape)
         for direction in args.directions.split(","):
             factory, kwargs = families[direction]
