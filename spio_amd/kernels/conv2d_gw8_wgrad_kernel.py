@@ -222,8 +222,8 @@ def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig, _dev
         defines.update(SPIO_PARTIALS=1)
         spec.workspace_bytes = num_partials * cols * 16
         spec.epilogue_suffix = "_reduce"
-        # one workgroup per 8 float4 columns (cols is a multiple of 8 per channel block)
-        spec.epilogue_launch_params = LaunchParams(grid=cols // 8, block=256)
+        # one workgroup per 32 float4 columns (cols is a multiple of 32 per channel block)
+        spec.epilogue_launch_params = LaunchParams(grid=cols // 32, block=256)
     return spec
 
 
