@@ -1,15 +1,25 @@
 """`spio::layernorm_2d`: LayerNorm over the channels of an NCHW tensor with channels_last strides.
 
 Forward runs the HIP kernel (csrc/layernorm_2d.hip; contract of the reference's
-spio/src/layernorm_2d.cu:81-222).  The backward pass is written with torch operations in fp32 on
-the same layout; it recomputes the statistics from the input.
+spio/src/layernorm_2d.cu:81-222).  The backward pass runs a second HIP kernel
+(csrc/layernorm_2d_bwd.hip: grad_input and per-workgroup partial sums of grad_weight and
+grad_bias in one pass over the input and grad_output, statistics recomputed from the input); the
+partial sums are added with one torch reduction.  Shapes that kernel does not take (more than
+1024 channels) and SPIO_LAYERNORM_BACKWARD=torch use torch operations in fp32 on the same layout.
 """
 
 from typing import Optional, Tuple
 
 import torch
 
-from ..kernels.layernorm_2d_kernel import LayerNorm2dParams, layernorm_2d_kernel_factory
+import os
+
+from ..kernels.layernorm_2d_kernel import (
+    LayerNorm2dParams,
+    layernorm_2d_bwd_is_supported,
+    layernorm_2d_bwd_kernel_factory,
+    layernorm_2d_kernel_factory,
+)
 
 
 @torch.library.custom_op("spio::layernorm_2d", mutates_args=())
@@ -46,8 +56,43 @@ def _setup_context(ctx, inputs, output):
     ctx.has_bias = bias is not None
 
 
+@torch.library.custom_op("spio::layernorm_2d_backward", mutates_args=())
+def layernorm_2d_backward(inputs: torch.Tensor, grad_output: torch.Tensor, weight: Optional[torch.Tensor],
+                          eps: float) -> Tuple[torch.Tensor, torch.Tensor]:  # fmt: skip
+    """(grad_input fp16, [grad_weight; grad_bias] fp32 as one [2, C] tensor) of layernorm_2d: one
+    kernel and one sum over the workgroups' partial rows."""
+    n, c, h, w = (int(v) for v in inputs.shape)
+    params = LayerNorm2dParams(n=n, c=c, h=h, w=w, eps=float(eps), has_weight=weight is not None, has_bias=False)
+    x = inputs.contiguous(memory_format=torch.channels_last)
+    dy = grad_output.to(torch.float16).contiguous(memory_format=torch.channels_last)
+    kernel = layernorm_2d_bwd_kernel_factory.get_kernel(params, inputs.device)
+    grid = kernel.kernel_spec.launch_params.grid[0]
+    grad_input = torch.empty_like(x, memory_format=torch.channels_last)
+    partials = torch.empty((grid, 2, c), dtype=torch.float32, device=inputs.device)
+    kernel(grad_input, partials, x, dy, None if weight is None else weight.detach().float().contiguous())
+    return grad_input, partials.sum(0)
+
+
+@layernorm_2d_backward.register_fake
+def _layernorm_2d_backward_fake(inputs, grad_output, weight, eps):
+    c = inputs.shape[1]
+    return (torch.empty_like(inputs, memory_format=torch.channels_last),
+            inputs.new_empty((2, c), dtype=torch.float32))  # fmt: skip
+
+
 def _backward(ctx, grad_output) -> Tuple[Optional[torch.Tensor], ...]:
     x, weight = ctx.saved_tensors
+    n, c, h, w = (int(v) for v in x.shape)
+    use_kernel = (os.environ.get("SPIO_LAYERNORM_BACKWARD", "hip") != "torch" and x.device.type == "cuda"
+                  and layernorm_2d_bwd_is_supported(LayerNorm2dParams(n=n, c=c, h=h, w=w)))  # fmt: skip
+    if use_kernel:
+        grad_input, sums = layernorm_2d_backward(x, grad_output, weight, ctx.eps)
+        return (
+            grad_input if ctx.needs_input_grad[0] else None,
+            sums[0].to(weight.dtype) if weight is not None and ctx.needs_input_grad[1] else None,
+            sums[1] if ctx.has_bias and ctx.needs_input_grad[2] else None,
+            None,
+        )
     xf = x.float().permute(0, 2, 3, 1)  # [n, h, w, c] view of the channels_last tensor
     dy = grad_output.float().permute(0, 2, 3, 1)
     mean = xf.mean(-1, keepdim=True)

@@ -18,4 +18,11 @@ from .conv2d_gw8_bgrad_kernel import (
     Conv2dGw8BgradConfig,
     bgrad_is_supported,
 )
-from .layernorm_2d_kernel import layernorm_2d_kernel_factory, LayerNorm2dParams, LayerNorm2dConfig
+from .layernorm_2d_kernel import (
+    layernorm_2d_kernel_factory,
+    layernorm_2d_bwd_kernel_factory,
+    layernorm_2d_bwd_is_supported,
+    LayerNorm2dParams,
+    LayerNorm2dConfig,
+    LayerNorm2dBwdConfig,
+)

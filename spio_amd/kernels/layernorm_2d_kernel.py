@@ -154,3 +154,97 @@ layernorm_2d_kernel_factory = KernelFactory(
     kernel_spec=_get_kernel_spec,
     make_test_args=_make_test_args,
 )
+
+
+# ---- backward: grad_input and per-workgroup partial sums of grad_weight / grad_bias ----
+#
+# Kernel arguments: (grad_input, partials, input, grad_output, weight or None); `partials` is an
+# fp32 workspace of [grid][2][C] that the kernel overwrites (row = workgroup, 0 = grad_weight,
+# 1 = grad_bias); its rows are summed by the caller.
+
+BWD_SOURCE = "layernorm_2d_bwd.hip"
+BWD_MAX_CHANNELS = 1024  # the workgroup's channel sums meet in LDS: waves x 2 x C floats
+BWD_MAX_GROUPS_PER_CU = 4
+
+
+@dataclass(frozen=True)
+class LayerNorm2dBwdConfig:
+    """As LayerNorm2dConfig; `unroll` counts pixel groups whose input and grad_output loads are
+    in flight together, and few workgroups per compute unit keep the partial sums few."""
+
+    threads: int = 256
+    unroll: int = 2
+    groups_per_cu: int = 2
+    lanes: int = 0
+
+
+def layernorm_2d_bwd_is_supported(params: LayerNorm2dParams) -> bool:
+    return params.c % 8 == 0 and params.c <= BWD_MAX_CHANNELS
+
+
+def _get_bwd_configs(params: LayerNorm2dParams, _device_attr=None) -> List[LayerNorm2dBwdConfig]:
+    if not layernorm_2d_bwd_is_supported(params):
+        return []
+    per_lanes = []
+    for lanes in _lane_choices(params.c):
+        upl = divup(params.c // 8, lanes or lanes_per_pixel(params.c))
+        mine = []
+        for threads in (256, 512):
+            for unroll in (4, 2, 1):
+                if unroll * upl > 4:
+                    continue
+                for per_cu in (2, 4, 1):
+                    mine.append(LayerNorm2dBwdConfig(threads, unroll, per_cu, lanes))
+        per_lanes.append(mine)
+    out = []
+    for i in range(max(len(m) for m in per_lanes)):
+        for mine in reversed(per_lanes):
+            if i < len(mine):
+                out.append(mine[i])
+    return out
+
+
+def _get_bwd_kernel_spec(params: LayerNorm2dParams, config: LayerNorm2dBwdConfig, device_attr=None) -> KernelSpec:
+    params.validate()
+    assert layernorm_2d_bwd_is_supported(params), f"unsupported shape {params}"
+    cus = getattr(device_attr, "multiprocessor_count", 256) or 256
+    lpp = config.lanes or lanes_per_pixel(params.c)
+    assert lpp & (lpp - 1) == 0 and lpp <= 64 and divup(params.c // 8, lpp) <= 4, f"illegal configuration {config}"
+    assert 1 <= config.groups_per_cu <= BWD_MAX_GROUPS_PER_CU
+    pass_pixels = (64 // lpp) * (config.threads // 64) * config.unroll
+    grid = max(1, min(divup(params.pixels, pass_pixels), cus * config.groups_per_cu))
+    defines = {
+        "SPIO_LN_C": params.c, "SPIO_LN_PIXELS": params.pixels, "SPIO_LN_LPP": lpp,
+        "SPIO_LN_THREADS": config.threads, "SPIO_LN_UNROLL": config.unroll,
+        "SPIO_LN_HAS_WEIGHT": int(params.has_weight),
+        "SPIO_LN_EPS": f"{params.eps:.9g}f", "SPIO_LN_GRID": grid,
+    }  # fmt: skip
+    return KernelSpec(defines, LaunchParams(grid=grid, block=config.threads), BWD_SOURCE,
+                      notes={"LPP": lpp, "PASS_PIXELS": pass_pixels, "GRID": grid})  # fmt: skip
+
+
+def layernorm_2d_bwd_partials(params: LayerNorm2dParams, device, device_attr=None) -> torch.Tensor:
+    """A workspace large enough for every configuration's partial sums (not initialised)."""
+    cus = getattr(device_attr, "multiprocessor_count", 256) or 256
+    return torch.empty((cus * BWD_MAX_GROUPS_PER_CU, 2, params.c), dtype=torch.float32, device=device)
+
+
+def _make_bwd_test_args(params: LayerNorm2dParams, device):
+    cl = torch.channels_last
+    x = torch.randn(params.shape, device=device, dtype=torch.float16).contiguous(memory_format=cl)
+    dy = torch.randn(params.shape, device=device, dtype=torch.float16).contiguous(memory_format=cl)
+    dx = torch.empty_like(x)
+    w = torch.randn(params.c, device=device, dtype=torch.float32) if params.has_weight else None
+    return (dx, layernorm_2d_bwd_partials(params, device), x, dy, w)
+
+
+layernorm_2d_bwd_kernel_factory = KernelFactory(
+    LayerNorm2dParams,
+    LayerNorm2dBwdConfig,
+    None,
+    kernel_name="spio_layernorm_2d_bwd",
+    configs=_get_bwd_configs,
+    kernel_spec=_get_bwd_kernel_spec,
+    make_test_args=_make_bwd_test_args,
+)
+

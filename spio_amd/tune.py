@@ -206,6 +206,8 @@ def main(argv=None):
         conv2d_gw8_bgrad_kernel_factory,
         conv2d_gw8_kernel_factory,
         conv2d_gw8_wgrad_kernel_factory,
+        layernorm_2d_bwd_is_supported,
+        layernorm_2d_bwd_kernel_factory,
         layernorm_2d_kernel_factory,
     )
     from .kernels.tuner import _PACKAGE_RECORDS, device_key, tuner
@@ -237,14 +239,20 @@ def main(argv=None):
         if shape in seen:
             continue
         seen.add(shape)
-        if "eps_" in shape:  # a LayerNorm2d shape: one kernel family, no directions
+        if "eps_" in shape:  # a LayerNorm2d shape: the forward kernel and the backward kernel
             params = LayerNorm2dParams.decode(shape)
-            kernel = tuner.sweep(layernorm_2d_kernel_factory, params, 0, attr, warmup=3, iters=args.iters,
-                                 record_path=path)  # fmt: skip
-            best = min(r["us"] for r in tuner.last_sweep if "us" in r)
-            print(f"lnorm {shape}: {best:8.1f} us  {kernel.config}", flush=True)
-            kernel.unload()
-            torch.cuda.empty_cache()
+            # the backward kernel does not depend on the bias: its records are kept without one
+            bwd_params = LayerNorm2dParams(n=params.n, c=params.c, h=params.h, w=params.w, eps=params.eps,
+                                           has_weight=params.has_weight, has_bias=False)  # fmt: skip
+            for tag, factory, p in (("lnorm", layernorm_2d_kernel_factory, params),
+                                    ("lnbwd", layernorm_2d_bwd_kernel_factory, bwd_params)):  # fmt: skip
+                if tag == "lnbwd" and not layernorm_2d_bwd_is_supported(p):
+                    continue
+                kernel = tuner.sweep(factory, p, 0, attr, warmup=3, iters=args.iters, record_path=path)
+                best = min(r["us"] for r in tuner.last_sweep if "us" in r)
+                print(f"{tag} {p.encode()}: {best:8.1f} us  {kernel.config}", flush=True)
+                kernel.unload()
+                torch.cuda.empty_cache()
             continue
         params = Conv2dGw8Params.decode(shape)
         for direction in args.directions.split(","):

@@ -155,7 +155,7 @@ def test_packaged_tuning_records_name_configurations_that_still_exist():
 
     import spio_amd.kernels as kernels_pkg
 
-    from spio_amd.kernels import LayerNorm2dParams, layernorm_2d_kernel_factory
+    from spio_amd.kernels import LayerNorm2dParams, layernorm_2d_bwd_kernel_factory, layernorm_2d_kernel_factory
 
     families = {
         "spio_conv2d_gw8_fprop": (conv2d_gw8_kernel_factory, {}),
@@ -163,6 +163,7 @@ def test_packaged_tuning_records_name_configurations_that_still_exist():
         "spio_conv2d_gw8_wgrad": (conv2d_gw8_wgrad_kernel_factory, {}),
         "spio_conv2d_gw8_bgrad": (conv2d_gw8_bgrad_kernel_factory, {}),
         "spio_layernorm_2d": (layernorm_2d_kernel_factory, {}),
+        "spio_layernorm_2d_bwd": (layernorm_2d_bwd_kernel_factory, {}),
     }
     tuned = os.path.join(os.path.dirname(kernels_pkg.__file__), "tuned")
     checked = 0
@@ -174,7 +175,7 @@ def test_packaged_tuning_records_name_configurations_that_still_exist():
         for key, record in records.items():
             name, encoded = key.split("__")
             factory, kw = families[name]
-            params = (LayerNorm2dParams if name == "spio_layernorm_2d" else Conv2dGw8Params).decode(encoded)
+            params = (LayerNorm2dParams if name.startswith("spio_layernorm_2d") else Conv2dGw8Params).decode(encoded)
             config = factory.config_cls(**record["config"])
             assert config in list(factory.configs(params, attr, **kw)), f"stale record {key}: {config}"
             assert record["us"] > 0

@@ -11,7 +11,12 @@ import torch.nn.functional as F
 
 from spio_amd.functional import layernorm_2d
 from spio_amd.hip import get_device_attributes
-from spio_amd.kernels import LayerNorm2dParams, layernorm_2d_kernel_factory
+from spio_amd.kernels import (
+    LayerNorm2dParams,
+    layernorm_2d_bwd_is_supported,
+    layernorm_2d_bwd_kernel_factory,
+    layernorm_2d_kernel_factory,
+)
 from spio_amd.layers import LayerNorm2d
 
 pytestmark = pytest.mark.gpu
@@ -61,6 +66,87 @@ def test_every_configuration_of_one_shape():
         torch.cuda.synchronize()
         torch.testing.assert_close(out.float().cpu(), expected, rtol=2e-3, atol=4e-3, msg=str(config))
         kernel.unload()
+
+
+def _reference_backward(x, dy, w, b, eps):
+    xr = x.float().requires_grad_(True)
+    wr = None if w is None else w.clone().requires_grad_(True)
+    br = None if b is None else b.clone().requires_grad_(True)
+    _reference(xr, wr, br, eps).backward(dy.float())
+    return xr.grad, None if wr is None else wr.grad, None if br is None else br.grad
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("affine", ["wb", "w", "none"])
+def test_layernorm_2d_backward_matches_torch(shape, affine):
+    """grad_input, grad_weight and grad_bias through the op's autograd (the backward kernel up to
+    1024 channels, torch operations beyond) against torch's autograd in fp32 on the CPU.
+    Tolerances: grad_input is one fp16 rounding of an O(1..10) value; the channel sums add up to
+    12544 products in fp32 in another order."""
+    g = torch.Generator().manual_seed(sum(shape) + 7)
+    x = (torch.randn(shape, generator=g) * 2 + 0.5).half()
+    dy = torch.randn(shape, generator=g).half()
+    c = shape[1]
+    w = torch.randn(c, generator=g) if affine != "none" else None
+    b = torch.randn(c, generator=g) if affine == "wb" else None
+    ex_dx, ex_dw, ex_db = _reference_backward(x, dy, w, b, 1e-6)
+    xg = x.cuda().contiguous(memory_format=torch.channels_last).requires_grad_(True)
+    wg = None if w is None else w.cuda().requires_grad_(True)
+    bg = None if b is None else b.cuda().requires_grad_(True)
+    out = layernorm_2d(xg, wg, bg, 1e-6)
+    out.backward(dy.cuda().contiguous(memory_format=torch.channels_last))
+    assert xg.grad.dtype == torch.float16
+    torch.testing.assert_close(xg.grad.float().cpu(), ex_dx, rtol=4e-3, atol=4e-3)
+    if w is not None:
+        torch.testing.assert_close(wg.grad.cpu(), ex_dw, rtol=2e-3, atol=3e-2)
+    if b is not None:
+        torch.testing.assert_close(bg.grad.cpu(), ex_db, rtol=2e-3, atol=3e-2)
+
+
+def test_every_backward_configuration_of_one_shape():
+    attr = get_device_attributes(0)
+    params = LayerNorm2dParams(n=3, c=192, h=13, w=11, has_bias=False)
+    assert layernorm_2d_bwd_is_supported(params)
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(params.shape, generator=g).half()
+    dy = torch.randn(params.shape, generator=g).half()
+    w = torch.randn(192, generator=g)
+    ex_dx, ex_dw, ex_db = _reference_backward(x, dy, w, torch.zeros(192), params.eps)
+    xg = x.cuda().contiguous(memory_format=torch.channels_last)
+    dyg = dy.cuda().contiguous(memory_format=torch.channels_last)
+    configs = layernorm_2d_bwd_kernel_factory.configs(params, attr)
+    assert {c.lanes for c in configs} == {0, 8}
+    for config in configs:
+        kernel = layernorm_2d_bwd_kernel_factory.make_kernel(params, config, attr)
+        kernel.compile()
+        kernel.load(0)
+        grid = kernel.kernel_spec.launch_params.grid[0]
+        dx = torch.full_like(xg, -42.0)
+        partials = torch.full((grid, 2, 192), float("nan"), device="cuda")
+        kernel(dx, partials, xg, dyg, w.cuda())
+        torch.cuda.synchronize()
+        torch.testing.assert_close(dx.float().cpu(), ex_dx, rtol=4e-3, atol=4e-3, msg=str(config))
+        sums = partials.sum(0).cpu()
+        torch.testing.assert_close(sums[0], ex_dw, rtol=2e-3, atol=3e-2, msg=str(config))
+        torch.testing.assert_close(sums[1], ex_db, rtol=2e-3, atol=3e-2, msg=str(config))
+        kernel.unload()
+
+
+def test_backward_falls_back_to_torch_operations(monkeypatch):
+    """SPIO_LAYERNORM_BACKWARD=torch takes the torch-operation backward; same gradients."""
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(2, 96, 6, 5, generator=g).half()
+    dy = torch.randn(2, 96, 6, 5, generator=g).half()
+    w, b = torch.randn(96, generator=g), torch.randn(96, generator=g)
+    grads = []
+    for mode in ("hip", "torch"):
+        monkeypatch.setenv("SPIO_LAYERNORM_BACKWARD", mode)
+        xg = x.cuda().contiguous(memory_format=torch.channels_last).requires_grad_(True)
+        wg, bg = w.cuda().requires_grad_(True), b.cuda().requires_grad_(True)
+        layernorm_2d(xg, wg, bg, 1e-6).backward(dy.cuda())
+        grads.append((xg.grad.float().cpu(), wg.grad.cpu(), bg.grad.cpu()))
+    for a, b_ in zip(*grads):
+        torch.testing.assert_close(a, b_, rtol=4e-3, atol=2e-2)
 
 
 def test_layer_and_backward():
