@@ -169,3 +169,18 @@ def test_layer_and_backward():
     torch.testing.assert_close(xg.grad.float().cpu(), xr.grad, rtol=4e-3, atol=4e-3)
     torch.testing.assert_close(layer.weight.grad.cpu(), wr.grad, rtol=2e-3, atol=2e-2)
     torch.testing.assert_close(layer.bias.grad.cpu(), br.grad, rtol=2e-3, atol=2e-2)
+
+
+def test_opcheck_forward_and_backward_ops():
+    """Schema, fake implementations (shapes, strides, dtypes) and autograd registration of both ops."""
+    from spio_amd.functional.layernorm_2d_function import layernorm_2d_backward
+
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(2, 48, 5, 6, generator=g).half().cuda().contiguous(memory_format=torch.channels_last)
+    dy = torch.randn(2, 48, 5, 6, generator=g).half().cuda().contiguous(memory_format=torch.channels_last)
+    w, b = torch.randn(48, generator=g).cuda(), torch.randn(48, generator=g).cuda()
+    torch.library.opcheck(layernorm_2d, (x.clone().requires_grad_(True), w.clone().requires_grad_(True),
+                                         b.clone().requires_grad_(True), 1e-6))  # fmt: skip
+    torch.library.opcheck(layernorm_2d_backward, (x, dy, w, 1e-6))
+    torch.library.opcheck(layernorm_2d_backward, (x, dy, None, 1e-6))
+
