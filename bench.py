@@ -616,7 +616,11 @@ def bench_network(args, device):
 
     from spio_amd.kernels import Conv2dGw8Params, Conv2dStats, conv2d_gw8_kernel_factory
     from spio_amd.layers import Conv2dGw8, LayerNorm2d
-    from spio_amd.kernels.layernorm_2d_kernel import LayerNorm2dParams, layernorm_2d_kernel_factory
+    from spio_amd.kernels.layernorm_2d_kernel import (
+        LayerNorm2dParams,
+        layernorm_2d_bwd_kernel_factory,
+        layernorm_2d_kernel_factory,
+    )
 
     batch = 128
     torch.manual_seed(3)
@@ -669,8 +673,20 @@ def bench_network(args, device):
         nsets = rotation_sets(nb)
         asets = [layernorm_2d_kernel_factory.make_test_args(p, device) for _ in range(nsets)]
         e = kernel_entry(k, asets, nb, 100)
-        norms.append({"shape": p.encode(), "us": e["us"], "GB/s": e["GB/s"],
-                      "frac_of_hbm_peak": e["frac_of_hbm_peak"], "bytes": nb})  # fmt: skip
+        entry = {"shape": p.encode(), "us": e["us"], "GB/s": e["GB/s"],
+                 "frac_of_hbm_peak": e["frac_of_hbm_peak"], "bytes": nb}  # fmt: skip
+        del asets
+        torch.cuda.empty_cache()
+        # its backward kernel (grad_input + partial sums of grad_weight / grad_bias): 4 B in, 2 B out
+        pb = LayerNorm2dParams(n=batch, c=c, h=hw, w=hw, has_bias=False)
+        kb = layernorm_2d_bwd_kernel_factory.get_kernel(pb, device)
+        nbb = 6 * batch * c * hw * hw + 4 * c
+        nsets = rotation_sets(nbb)
+        asets = [layernorm_2d_bwd_kernel_factory.make_test_args(pb, device) for _ in range(nsets)]
+        eb = kernel_entry(kb, asets, nbb, 100)
+        entry["backward"] = {"us": eb["us"], "GB/s": eb["GB/s"], "frac_of_hbm_peak": eb["frac_of_hbm_peak"],
+                             "bytes": nbb}  # fmt: skip
+        norms.append(entry)
         del asets
         torch.cuda.empty_cache()
     value = total_bytes / (total_us * 1e-6) / 1e9
