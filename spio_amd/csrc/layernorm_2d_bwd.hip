@@ -14,8 +14,9 @@
 // xor butterfly, the waves through LDS, and the workgroup writes one row of
 // `partials[workgroup][2][C]` with plain stores: every row is written completely, so the
 // workspace needs no zeroing and nothing is atomic (with atomics every workgroup would add to the
-// same C addresses, one after the other); the rows are summed by the caller.  HBM-bound: 4 bytes
-// in, 2 bytes out per element.
+// same C addresses, one after the other).  The small <name>_reduce kernel below adds the rows
+// into `sums[2][C]` (0 = grad_weight, 1 = grad_bias), which it overwrites.  HBM-bound: 4 bytes in,
+// 2 bytes out per element.
 #ifndef SPIO_LN_C
 #error "SPIO_LN_C, SPIO_LN_PIXELS, SPIO_LN_LPP, SPIO_LN_THREADS, SPIO_LN_GRID are required"
 #endif
@@ -83,7 +84,7 @@ __device__ inline float channel_sum(float v) {
 }  // namespace
 
 extern "C" __global__ void __attribute__((amdgpu_flat_work_group_size(THREADS, THREADS)))
-SPIO_KERNEL_NAME(ln_uint4* __restrict__ din, float* __restrict__ partials, const ln_uint4* __restrict__ in,
+SPIO_KERNEL_NAME(float* __restrict__ partials, ln_uint4* __restrict__ din, const ln_uint4* __restrict__ in,
                  const ln_uint4* __restrict__ dout, const float* __restrict__ weight) {
     constexpr long long num_workgroups = SPIO_LN_GRID;
     __shared__ float red[WAVES][2][LPP * UPL * 8];
@@ -216,3 +217,44 @@ SPIO_KERNEL_NAME(ln_uint4* __restrict__ din, float* __restrict__ partials, const
         row[i] = v;
     }
 }
+
+// Second stage: sums[i] = sum over the workgroups' rows of partials[row][i], i < 2*C.  A workgroup
+// owns 32 columns; its 8 slices each add the rows r = slice, slice + 8, ... with 8 loads in
+// flight, and meet in LDS.  Every element has one owner: no atomics, no dependence on timing.
+#define SPIO_LN_CONCAT2(a, b) a##b
+#define SPIO_LN_CONCAT(a, b) SPIO_LN_CONCAT2(a, b)
+extern "C" __global__ void __attribute__((amdgpu_flat_work_group_size(256, 256)))
+SPIO_LN_CONCAT(SPIO_KERNEL_NAME, _reduce)(float* __restrict__ sums, const float* __restrict__ partials) {
+    constexpr int ROWS = SPIO_LN_GRID;
+    constexpr int COLS = 32;
+    constexpr int SLICES = 256 / COLS;
+    constexpr int UNR = 8;
+    __shared__ float red[SLICES][COLS];
+    const int tid = (int)__builtin_amdgcn_workitem_id_x();
+    const int cl = tid % COLS;
+    const int slice = tid / COLS;
+    const int col = (int)__builtin_amdgcn_workgroup_id_x() * COLS + cl;
+    float sum = 0.f;
+    if (col < 2 * C) {
+        for (int base = slice; base < ROWS; base += SLICES * UNR) {
+            float v[UNR];
+#pragma unroll
+            for (int i = 0; i < UNR; ++i) {
+                const int r = base + i * SLICES;
+                v[i] = r < ROWS ? partials[(long long)r * 2 * C + col] : 0.f;
+            }
+#pragma unroll
+            for (int i = 0; i < UNR; ++i) sum += v[i];
+        }
+    }
+    red[slice][cl] = sum;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    if (slice == 0 && col < 2 * C) {
+#pragma unroll
+        for (int i = 1; i < SLICES; ++i) sum += red[i][cl];
+        sums[col] = sum;
+    }
+}
+

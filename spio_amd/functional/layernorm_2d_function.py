@@ -3,8 +3,8 @@
 Forward runs the HIP kernel (csrc/layernorm_2d.hip; contract of the reference's
 spio/src/layernorm_2d.cu:81-222).  The backward pass runs a second HIP kernel
 (csrc/layernorm_2d_bwd.hip: grad_input and per-workgroup partial sums of grad_weight and
-grad_bias in one pass over the input and grad_output, statistics recomputed from the input); the
-partial sums are added with one torch reduction.  Shapes that kernel does not take (more than
+grad_bias in one pass over the input and grad_output, statistics recomputed from the input, and a
+small second stage that adds the partial sums).  Shapes that kernel does not take (more than
 1024 channels) and SPIO_LAYERNORM_BACKWARD=torch use torch operations in fp32 on the same layout.
 """
 
@@ -59,18 +59,17 @@ def _setup_context(ctx, inputs, output):
 @torch.library.custom_op("spio::layernorm_2d_backward", mutates_args=())
 def layernorm_2d_backward(inputs: torch.Tensor, grad_output: torch.Tensor, weight: Optional[torch.Tensor],
                           eps: float) -> Tuple[torch.Tensor, torch.Tensor]:  # fmt: skip
-    """(grad_input fp16, [grad_weight; grad_bias] fp32 as one [2, C] tensor) of layernorm_2d: one
-    kernel and one sum over the workgroups' partial rows."""
+    """(grad_input fp16, [grad_weight; grad_bias] fp32 as one [2, C] tensor) of layernorm_2d: the
+    backward kernel and its small second stage that adds the workgroups' partial rows."""
     n, c, h, w = (int(v) for v in inputs.shape)
     params = LayerNorm2dParams(n=n, c=c, h=h, w=w, eps=float(eps), has_weight=weight is not None, has_bias=False)
     x = inputs.contiguous(memory_format=torch.channels_last)
     dy = grad_output.to(torch.float16).contiguous(memory_format=torch.channels_last)
     kernel = layernorm_2d_bwd_kernel_factory.get_kernel(params, inputs.device)
-    grid = kernel.kernel_spec.launch_params.grid[0]
     grad_input = torch.empty_like(x, memory_format=torch.channels_last)
-    partials = torch.empty((grid, 2, c), dtype=torch.float32, device=inputs.device)
-    kernel(grad_input, partials, x, dy, None if weight is None else weight.detach().float().contiguous())
-    return grad_input, partials.sum(0)
+    sums = torch.empty((2, c), dtype=torch.float32, device=inputs.device)
+    kernel(sums, grad_input, x, dy, None if weight is None else weight.detach().float().contiguous())
+    return grad_input, sums
 
 
 @layernorm_2d_backward.register_fake

@@ -158,9 +158,10 @@ layernorm_2d_kernel_factory = KernelFactory(
 
 # ---- backward: grad_input and per-workgroup partial sums of grad_weight / grad_bias ----
 #
-# Kernel arguments: (grad_input, partials, input, grad_output, weight or None); `partials` is an
-# fp32 workspace of [grid][2][C] that the kernel overwrites (row = workgroup, 0 = grad_weight,
-# 1 = grad_bias); its rows are summed by the caller.
+# Kernel arguments: (sums, grad_input, input, grad_output, weight or None); `sums` is fp32 [2][C]
+# (0 = grad_weight, 1 = grad_bias) and is overwritten.  Two stages: the main kernel writes one row
+# of partial sums per workgroup into a workspace of [grid][2][C] floats, the <name>_reduce kernel
+# adds the rows.
 
 BWD_SOURCE = "layernorm_2d_bwd.hip"
 BWD_MAX_CHANNELS = 1024  # the workgroup's channel sums meet in LDS: waves x 2 x C floats
@@ -219,14 +220,12 @@ def _get_bwd_kernel_spec(params: LayerNorm2dParams, config: LayerNorm2dBwdConfig
         "SPIO_LN_HAS_WEIGHT": int(params.has_weight),
         "SPIO_LN_EPS": f"{params.eps:.9g}f", "SPIO_LN_GRID": grid,
     }  # fmt: skip
-    return KernelSpec(defines, LaunchParams(grid=grid, block=config.threads), BWD_SOURCE,
+    spec = KernelSpec(defines, LaunchParams(grid=grid, block=config.threads), BWD_SOURCE,
                       notes={"LPP": lpp, "PASS_PIXELS": pass_pixels, "GRID": grid})  # fmt: skip
-
-
-def layernorm_2d_bwd_partials(params: LayerNorm2dParams, device, device_attr=None) -> torch.Tensor:
-    """A workspace large enough for every configuration's partial sums (not initialised)."""
-    cus = getattr(device_attr, "multiprocessor_count", 256) or 256
-    return torch.empty((cus * BWD_MAX_GROUPS_PER_CU, 2, params.c), dtype=torch.float32, device=device)
+    spec.workspace_bytes = grid * 2 * params.c * 4
+    spec.epilogue_suffix = "_reduce"
+    spec.epilogue_launch_params = LaunchParams(grid=divup(2 * params.c, 32), block=256)
+    return spec
 
 
 def _make_bwd_test_args(params: LayerNorm2dParams, device):
@@ -235,7 +234,8 @@ def _make_bwd_test_args(params: LayerNorm2dParams, device):
     dy = torch.randn(params.shape, device=device, dtype=torch.float16).contiguous(memory_format=cl)
     dx = torch.empty_like(x)
     w = torch.randn(params.c, device=device, dtype=torch.float32) if params.has_weight else None
-    return (dx, layernorm_2d_bwd_partials(params, device), x, dy, w)
+    sums = torch.empty((2, params.c), device=device, dtype=torch.float32)
+    return (sums, dx, x, dy, w)
 
 
 layernorm_2d_bwd_kernel_factory = KernelFactory(

@@ -274,10 +274,11 @@ class Tuner:
         """Run `kernel` once on copies of the synthetic arguments; returns its output tensors."""
         import torch  # pylint: disable=import-outside-toplevel
 
-        # outputs come first in every kernel family here: (dst, ...), (dw, ...), (dx, dw, ...);
-        # the gradient kernels of a layer with a bias take grad_bias as their last argument
+        # outputs come first in every kernel family here: (dst, ...), (dw, ...), (dx, dw, ...),
+        # (sums, dx, ...); the gradient kernels of a layer with a bias take grad_bias as their
+        # last argument
         family = kernel.kernel_name.split("__")[0]
-        n_out = 2 if family.endswith("bgrad") else 1
+        n_out = 2 if family.endswith(("bgrad", "_bwd")) else 1
         trailing_out = family.endswith(("wgrad", "bgrad")) and getattr(params, "has_bias", False)
         call = list(args)
         outs = []
