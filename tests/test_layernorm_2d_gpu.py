@@ -183,3 +183,46 @@ def test_opcheck_forward_and_backward_ops():
     torch.library.opcheck(layernorm_2d_backward, (x, dy, w, 1e-6))
     torch.library.opcheck(layernorm_2d_backward, (x, dy, None, 1e-6))
 
+
+def test_ops_replay_correctly_from_a_hip_graph():
+    """Forward and backward ops captured once into a HIP graph and replayed three times on new
+    data, with eager work and synchronisations between the replays; every replay must match the
+    eager reference (both ops launch their own kernels only: no library reduction, no memset)."""
+    from spio_amd.functional.layernorm_2d_function import layernorm_2d_backward
+
+    g = torch.Generator().manual_seed(11)
+    shape = (3, 192, 9, 10)
+    x = torch.empty(shape, dtype=torch.float16, device="cuda").contiguous(memory_format=torch.channels_last)
+    dy = torch.empty_like(x)
+    w = torch.randn(192, generator=g).cuda()
+    b = torch.randn(192, generator=g).cuda()
+
+    def run():
+        y = layernorm_2d(x, w, b, 1e-6)
+        dx, sums = layernorm_2d_backward(x, dy, w, 1e-6)
+        return y, dx, sums
+
+    x.normal_(), dy.normal_()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()  # first use outside the capture: kernel compilation and loading
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            outs = run()
+    torch.cuda.current_stream().wait_stream(side)
+    for trial in range(3):
+        xt = (torch.randn(shape, generator=g) * 2 + 0.5).half()
+        dyt = torch.randn(shape, generator=g).half()
+        x.copy_(xt.cuda()), dy.copy_(dyt.cuda())
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        ex_y = _reference(xt, w.cpu(), b.cpu(), 1e-6)
+        ex_dx, ex_dw, ex_db = _reference_backward(xt, dyt, w.cpu(), b.cpu(), 1e-6)
+        msg = f"graph replay {trial}"
+        torch.testing.assert_close(outs[0].float().cpu(), ex_y, rtol=2e-3, atol=4e-3, msg=msg)
+        torch.testing.assert_close(outs[1].float().cpu(), ex_dx, rtol=4e-3, atol=4e-3, msg=msg)
+        torch.testing.assert_close(outs[2][0].cpu(), ex_dw, rtol=2e-3, atol=3e-2, msg=msg)
+        torch.testing.assert_close(outs[2][1].cpu(), ex_db, rtol=2e-3, atol=3e-2, msg=msg)
+
