@@ -48,11 +48,18 @@ def test_scan_modules_reports_params():
 
 @pytest.mark.gpu
 def test_transformed_model_matches_original():
+    """The transformed model on the GPU against the original model in fp32 on the CPU (torch's
+    host convolution, the oracle's own reference), not against the GPU library's convolution."""
+    import copy
+
     torch.manual_seed(0)
-    model = Block().cuda().to(memory_format=torch.channels_last)
+    cpu_model = Block().float()
+    model = copy.deepcopy(cpu_model).cuda().to(memory_format=torch.channels_last)
     new = transform(model)
-    x = torch.randn(2, 3, 16, 16, device="cuda").contiguous(memory_format=torch.channels_last)
-    with torch.autocast(device_type="cuda", dtype=torch.float16):
-        got = new(x)
-        want = model(x)
-    assert torch.allclose(got.float(), want.float(), rtol=2e-3, atol=2e-2)
+    x = torch.randn(2, 3, 16, 16)
+    with torch.no_grad():
+        want = cpu_model(x)
+        with torch.autocast(device_type="cuda", dtype=torch.float16):
+            got = new(x.cuda().contiguous(memory_format=torch.channels_last))
+    # fp16 activations between the layers: a few roundings of O(1) values
+    torch.testing.assert_close(got.float().cpu(), want, rtol=1e-2, atol=2e-2)
