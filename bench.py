@@ -624,8 +624,9 @@ def bench_network(args, device):
 
     batch = 128
     torch.manual_seed(3)
+    # eps = 1e-6 as in ConvNeXt: the LayerNorm shapes the packaged tuning records cover
     model = ConvNeXtGw8(make_conv=lambda dim: Conv2dGw8(dim, dim, 3, padding=1, groups=dim // 8),
-                        norm2d=LayerNorm2d)  # fmt: skip
+                        norm2d=lambda dim: LayerNorm2d(dim, eps=1e-6))  # fmt: skip
     model = model.to(device).to(memory_format=torch.channels_last).eval()  # fp32 parameters, fp16 autocast
     gen = torch.Generator().manual_seed(3)
     images = [torch.randn(batch, 3, 224, 224, generator=gen).half().to(device)
