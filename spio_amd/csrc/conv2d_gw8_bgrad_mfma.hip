@@ -12,15 +12,19 @@
 // 2*|dy| + |x| + |dx| bytes through HBM; fused, dy is read once: 25 % less traffic for the
 // backward step of an HBM-bound operator, and one launch instead of two.
 //
-// Scope: "same" convolutions only (2*py = R-1, 2*px = S-1, so P = H and Q = W): then one copy
-// of a dy row in LDS serves both gradients, and the dx row that completes at a step has the
-// index of the x row of that step.  A workgroup owns SPIO_BH rows (of dx, and of dy for the
-// weight gradient) of SPIO_NB images side by side for SPIO_GB channel groups, repeated for
-// SPIO_ITERS image blocks.  It streams the rows p0-py .. p0+BH-1+py of dy and of x: step t
+// Scope: odd filter sizes.  The kernel computes a "same" convolution (2*py = R-1, 2*px = S-1, so
+// P = H and Q = W): then one copy of a dy row in LDS serves both gradients, and the dx row that
+// completes at a step has the index of the x row of that step.  Any other padding of an odd
+// filter is that convolution on a larger domain, DH = max(H, P) by DW = max(W, Q), in which the
+// smaller of x and dy sits centred with zeros around it: only the global addressing knows the
+// tensors' real extents (domain rows and columns outside a tensor load zeros and store nothing),
+// and below "row", "column", py and px are the domain's.
+// A workgroup owns SPIO_BH rows (of dx, and of dy for the weight gradient) of SPIO_NB images
+// side by side for SPIO_GB channel groups, repeated for SPIO_ITERS image blocks.  It streams the rows p0-py .. p0+BH-1+py of dy and of x: step t
 // stages dy row p0-py+t and x row p0-2py+t (an x row can only be multiplied once the dy rows
 // up to py below it are there).  The py halo rows of dy above and below the block feed the
 // data gradient only; the weight gradient masks them out of its dy fragments, so every dy row
-// is counted by exactly one workgroup.  With SPIO_BH = P a workgroup owns whole images and
+// is counted by exactly one workgroup.  With SPIO_BH = DH a workgroup owns whole images and
 // there is no halo.  Everything else is the separate kernels' design:
 //   * rows of x and dy staged in LDS as [group][flattened pixel][8 ch], zero halo materialised
 //     once, branch-free global loads SPIO_PF steps ahead;
@@ -69,7 +73,18 @@ using namespace spio;
 
 namespace {
 
-static_assert(2 * kPadY == kR - 1 && 2 * kPadX == kS - 1, "the fused backward kernel needs P = H and Q = W");
+static_assert(kR % 2 == 1 && kS % 2 == 1, "the fused backward kernel needs odd filter sizes");
+
+// The kernel works on a size-preserving convolution of DH x DW images with the padding
+// (PYS, PXS); x (and dx) and dy sit inside that domain at the offsets (XOY, XOX) and (DOY, DOX),
+// one of each pair being 0, and count as zero around their real extent.
+constexpr int PYS = (kR - 1) / 2;
+constexpr int PXS = (kS - 1) / 2;
+constexpr int DH = kH > kP ? kH : kP;
+constexpr int DW = kW > kQ ? kW : kQ;
+constexpr int XOY = (DH - kH) / 2, XOX = (DW - kW) / 2;
+constexpr int DOY = (DH - kP) / 2, DOX = (DW - kQ) / 2;
+static_assert(DOY - XOY == PYS - kPadY && DOX - XOX == PXS - kPadX, "domain offsets");
 
 constexpr int GB = SPIO_GB;        // groups per workgroup
 constexpr int BH = SPIO_BH;        // rows per workgroup
@@ -86,9 +101,9 @@ constexpr int S2 = 2 * ((kS + 1) / 2);
 constexpr int NBLK = S2 / 2;          // column-tap pairs
 constexpr int ND = kR + 1;            // values of delta
 constexpr int NPAIR = kR / 2 + 1;     // aligned dy row pairs one x row meets
-constexpr int WPI = kW + kS - 1;      // padded width of one image
+constexpr int WPI = DW + kS - 1;      // padded width of one image
 constexpr int F = NB * WPI;           // flattened pixels of a staged row
-constexpr int KSPAN = (NB - 1) * WPI + kQ;
+constexpr int KSPAN = (NB - 1) * WPI + DW;
 constexpr int KC = (KSPAN + 31) / 32;     // 32-pixel chunks
 constexpr int CPW = (KC + TS - 1) / TS;   // chunks per wave
 // ---- data gradient ----
@@ -100,7 +115,7 @@ constexpr int TPW = (WT + TS - 1) / TS;      // tiles per wave
 // ---- LDS geometry ----
 constexpr int FPX = 32 * KC + S2 - 1;  // x pixels a weight-gradient read can touch
 constexpr int GSX = FPX + ((9 - FPX % 16) + 16) % 16;  // x group stride (pixels), = 9 mod 16
-constexpr int FPD_W = kPadX + 32 * KC;                 // dy pixels: weight-gradient reads
+constexpr int FPD_W = PXS + 32 * KC;                   // dy pixels: weight-gradient reads
 constexpr int FPD_D = 16 * WT + 4 * KB - 1;            // dy pixels: data-gradient reads
 constexpr int FPD = FPD_W > FPD_D ? FPD_W : FPD_D;
 constexpr int GSD = FPD + ((9 - FPD % 16) + 16) % 16;  // dy group stride, = 9 mod 16
@@ -119,16 +134,16 @@ constexpr int OSTRIDE = GB * 16 + 16;        // bytes per pixel in the dx output
 constexpr int OUT_ROW_BYTES = 16 * WT * OSTRIDE;
 constexpr int X_CELLS = F * GB;
 constexpr int LPTX = (X_CELLS + THREADS - 1) / THREADS;
-constexpr int D_CELLS = NB * kQ * GB;
+constexpr int D_CELLS = NB * DW * GB;
 constexpr int LPTD = (D_CELLS + THREADS - 1) / THREADS;  // dy loads = dx stores per thread per row
 constexpr int GBLKS = (kGroups + GB - 1) / GB;
 constexpr int NBLKS = (kN + NB * ITERS - 1) / (NB * ITERS);
-constexpr int PBLKS = (kP + BH - 1) / BH;
+constexpr int PBLKS = (DH + BH - 1) / BH;
 constexpr int NUM_BLOCKS = GBLKS * PBLKS * NBLKS;
 // steps: dy rows p0-py .. p0+BH-1+py, then py more for the last x rows.  The bias sum takes a dy
 // row pair one step after its first row was staged, so a one-row filter needs one more step
 // when the sum is wanted.
-constexpr int ROWS = BH + 3 * kPadY + (SPIO_HAS_BIAS && kR == 1 ? 1 : 0);
+constexpr int ROWS = BH + 3 * PYS + (SPIO_HAS_BIAS && kR == 1 ? 1 : 0);
 
 constexpr int gcd_(int a, int b) { return b == 0 ? a : gcd_(b, a % b); }
 constexpr int LCM = NS / gcd_(NS, PF) * PF;  // lcm(NS, PF): even
@@ -154,9 +169,12 @@ constexpr int LDS_UNITS = max3(STREAM_UNITS, FILTER_UNITS, (PUBLISH_FLOATS + 3) 
 static_assert(LDS_UNITS * 16 <= 160 * 1024, "LDS overflow");
 static_assert(PF >= 2 && PF % 2 == 0 && WAVES <= 16, "bad configuration");
 
-constexpr long long IMAGE_BYTES = (long long)kH * kW * kC * 2;  // of x, dy and dx alike
-static_assert(NB * IMAGE_BYTES < (1ll << 31), "an image block must stay below 2 GiB (32-bit buffer offsets)");
-constexpr int ROW_BYTES = kW * kC * 2;
+constexpr long long X_IMAGE_BYTES = (long long)kH * kW * kC * 2;  // of x and dx
+constexpr long long D_IMAGE_BYTES = (long long)kP * kQ * kC * 2;  // of dy
+static_assert(NB * X_IMAGE_BYTES < (1ll << 31) && NB * D_IMAGE_BYTES < (1ll << 31),
+              "an image block must stay below 2 GiB (32-bit buffer offsets)");
+constexpr int X_ROW_BYTES = kW * kC * 2;
+constexpr int D_ROW_BYTES = kQ * kC * 2;
 constexpr unsigned OOB = 0x80000000u;  // offset of a lane without data: beyond every descriptor
 constexpr int AUX_NT = SPIO_NT ? 2 : 0;
 
@@ -224,10 +242,10 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
     const int cb = kSplitLines ? b % GBLKS : (b / PBLKS) % GBLKS;
     const int nbk = b / (PBLKS * GBLKS);
     const int p0 = pb * BH;
-    const int bh_eff = imin(BH, kP - p0);  // rows this block owns
-    // first and last row (of x and of dy alike) the block needs; loads outside repeat them
-    const int row_lo = imax(p0 - kPadY, 0);
-    const int row_hi = imin(p0 + bh_eff - 1 + kPadY, kP - 1);
+    const int bh_eff = imin(BH, DH - p0);  // rows this block owns
+    // first and last row (of the domain: of x and of dy alike) the block needs
+    const int row_lo = imax(p0 - PYS, 0);
+    const int row_hi = imin(p0 + bh_eff - 1 + PYS, DH - 1);
     const int gglob = cb * GB + wg;
     const bool wave_active = gglob < kGroups;
 
@@ -285,7 +303,7 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
     const int tt = lane & 3;
     const int sel = tt >> 1;
     const int xfrag_off = ((wg * GSX + 8 * kb + jr + sel) * 16) + (tt & 1) * 8;
-    const int dfrag_off = ((wg * GSD + kPadX + 8 * kb + jr) * 16) + (tt & 1) * 8;
+    const int dfrag_off = ((wg * GSD + PXS + 8 * kb + jr) * 16) + (tt & 1) * 8;
     // data gradient: D[m = 4*(lane/16)+i][n = lane%16]: pixel n, row slot lane/32, channels
     // 4*((lane/16)&1) + i
     const int out_j = lane >> 5;
@@ -311,12 +329,12 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
         // ---- buffer descriptors of this image block; images past the end of the batch lie
         //      beyond their size ----
         const int images = imin(NB, kN - n0);
-        const rsrc_t rs_x = make_rsrc(reinterpret_cast<const unsigned char*>(x) + n0 * IMAGE_BYTES,
-                                      (int)(images * IMAGE_BYTES));
-        const rsrc_t rs_dy = make_rsrc(reinterpret_cast<const unsigned char*>(dy) + n0 * IMAGE_BYTES,
-                                       (int)(images * IMAGE_BYTES));
-        const rsrc_t rs_dx = make_rsrc(reinterpret_cast<const unsigned char*>(grad_input) + n0 * IMAGE_BYTES,
-                                       (int)(images * IMAGE_BYTES));
+        const rsrc_t rs_x = make_rsrc(reinterpret_cast<const unsigned char*>(x) + n0 * X_IMAGE_BYTES,
+                                      (int)(images * X_IMAGE_BYTES));
+        const rsrc_t rs_dy = make_rsrc(reinterpret_cast<const unsigned char*>(dy) + n0 * D_IMAGE_BYTES,
+                                       (int)(images * D_IMAGE_BYTES));
+        const rsrc_t rs_dx = make_rsrc(reinterpret_cast<const unsigned char*>(grad_input) + n0 * X_IMAGE_BYTES,
+                                       (int)(images * X_IMAGE_BYTES));
 
         // ---- loop-invariant addressing (cells without data carry the out-of-range offset: they
         //      load zeros, which is what halo and gap cells must hold) ----
@@ -331,38 +349,45 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                 const int g = cell % GB;
                 const int f = cell / GB;
                 const int img = f / WPI;
-                const int col = f % WPI - kPadX;
+                const int col = f % WPI - PXS - XOX;  // column of x
                 x_lds[l] = g * GSX + f;
                 if (col >= 0 && col < kW && cb * GB + g < kGroups)
                     x_voff[l] = (unsigned)(((img * kH * kW + col) * kGroups + cb * GB + g) * 16);
             }
         }
-        // dy cells, and the dx cells of the same (image, column, group): same offset
-        unsigned d_voff[LPTD];
+        // dy cells, and the dx cells of the same (image, domain column, group): where dy and x have
+        // the same size, the same offset
+        unsigned d_voff[LPTD], o_voff[LPTD];
         int d_lds[LPTD], o_lds[LPTD];
 #pragma unroll
         for (int l = 0; l < LPTD; ++l) {
             const int cell = tid + THREADS * l;
             d_voff[l] = OOB;
+            o_voff[l] = OOB;
             d_lds[l] = DDUMP;
             o_lds[l] = 0;
             if (cell < D_CELLS) {
                 const int g = cell % GB;
-                const int q = (cell / GB) % kQ;
-                const int img = cell / (GB * kQ);
-                d_lds[l] = g * GSD + img * WPI + q + kPadX;
+                const int q = (cell / GB) % DW;
+                const int img = cell / (GB * DW);
+                d_lds[l] = g * GSD + img * WPI + q + PXS;
                 o_lds[l] = (img * WPI + q) * OSTRIDE + g * 16;
-                if (cb * GB + g < kGroups)
-                    d_voff[l] = (unsigned)(((img * kP * kQ + q) * kGroups + cb * GB + g) * 16);
+                const int qd = q - DOX;  // column of dy
+                const int wx = q - XOX;  // column of dx
+                if (qd >= 0 && qd < kQ && cb * GB + g < kGroups)
+                    d_voff[l] = (unsigned)(((img * kP * kQ + qd) * kGroups + cb * GB + g) * 16);
+                if (wx >= 0 && wx < kW && cb * GB + g < kGroups)
+                    o_voff[l] = (unsigned)(((img * kH * kW + wx) * kGroups + cb * GB + g) * 16);
             }
         }
 
-        // Rows `t` of x (image row p0-2py+t) and of dy (p0-py+t) for every cell of the thread.
-        // Rows the block does not need read through the empty descriptor (zeros, no traffic).
+        // Rows `t` of x (domain row p0-2py+t) and of dy (p0-py+t) for every cell of the thread.
+        // Rows the block does not need, and domain rows outside the tensor, read through the empty
+        // descriptor (zeros, no traffic).
         auto load_rows = [&](spio_uint4(&xr)[LPTX], spio_uint4(&dr)[LPTD], int t) {
-            const int h = p0 - 2 * kPadY + t;
-            const rsrc_t rx = (h >= row_lo && h <= row_hi) ? rs_x : rs_none;
-            const int sx = __builtin_amdgcn_readfirstlane(imin(imax(h, 0), kH - 1) * ROW_BYTES);
+            const int h = p0 - 2 * PYS + t;
+            const rsrc_t rx = (h >= row_lo && h <= row_hi && h >= XOY && h < XOY + kH) ? rs_x : rs_none;
+            const int sx = __builtin_amdgcn_readfirstlane(imin(imax(h - XOY, 0), kH - 1) * X_ROW_BYTES);
             const bool xhalo = h < p0 || h >= p0 + bh_eff;
 #pragma unroll
             for (int l = 0; l < LPTX; ++l) {
@@ -371,9 +396,9 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                                                   : __builtin_amdgcn_raw_buffer_load_b128(rx, (int)x_voff[l], sx, AUX_NT);
                 xr[l] = v.u;
             }
-            const int pr = p0 - kPadY + t;
-            const rsrc_t rd = (pr >= row_lo && pr <= row_hi) ? rs_dy : rs_none;
-            const int sd = __builtin_amdgcn_readfirstlane(imin(imax(pr, 0), kP - 1) * ROW_BYTES);
+            const int pr = p0 - PYS + t;
+            const rsrc_t rd = (pr >= row_lo && pr <= row_hi && pr >= DOY && pr < DOY + kP) ? rs_dy : rs_none;
+            const int sd = __builtin_amdgcn_readfirstlane(imin(imax(pr - DOY, 0), kP - 1) * D_ROW_BYTES);
             const bool dhalo = pr < p0 || pr >= p0 + bh_eff;
 #pragma unroll
             for (int l = 0; l < LPTD; ++l) {
@@ -407,12 +432,13 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
 #pragma unroll
             for (int a = 0; a < NACC; ++a) dacc[i][a] = spio_float4{0.f, 0.f, 0.f, 0.f};
 
-        // Coalesced store of the dx row staged at step `ts` (row p0 - 2py + ts), one step later.
-        // Steps that finish no row of the block store through the empty descriptor: the
+        // Coalesced store of the dx row staged at step `ts` (domain row p0 - 2py + ts), one step
+        // later.  Steps that finish no row of the block, or a domain row outside dx, store through
+        // the empty descriptor: the
         // instructions are issued all the same and the hardware drops them.
         auto store_dx_row = [&](int ts, int obuf) {
-            const int h = p0 - 2 * kPadY + ts;
-            const bool real = ts >= 2 * kPadY && ts < 2 * kPadY + bh_eff;
+            const int h = p0 - 2 * PYS + ts;
+            const bool real = ts >= 2 * PYS && ts < 2 * PYS + bh_eff && h >= XOY && h < XOY + kH;
             const rsrc_t rs = real ? rs_dx : rs_none;
             // The row offset is added to the per-lane offset; the scalar-offset operand stays the
             // constant 0.  A 16-byte buffer store reads its data registers for a few cycles after
@@ -420,12 +446,12 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
             // instructions from writing them: with the row offset in a scalar register a result
             // moved into the first data register right behind the store was stored in its place
             // (seen on gfx950 as stray values in the first two channels of some pixels).
-            const unsigned row_off = (unsigned)(imin(imax(h, 0), kH - 1) * ROW_BYTES);
+            const unsigned row_off = (unsigned)(imin(imax(h - XOY, 0), kH - 1) * X_ROW_BYTES);
 #pragma unroll
             for (int l = 0; l < LPTD; ++l) {
                 Pack16 v;
                 v.u = *reinterpret_cast<const spio_uint4*>(ostage + obuf * OUT_ROW_BYTES + o_lds[l]);
-                __builtin_amdgcn_raw_buffer_store_b128(v.i, rs, (int)(d_voff[l] + row_off), 0, AUX_NT);
+                __builtin_amdgcn_raw_buffer_store_b128(v.i, rs, (int)(o_voff[l] + row_off), 0, AUX_NT);
             }
         };
 
@@ -442,12 +468,12 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                 // 1. fragment reads: x row p0-2py+t, the dy row pairs it meets (dy rows are named
                 //    by the step that staged them: row p0-py+tau at step tau; the block owns
                 //    tau in [py, py+bh_eff)), and dy row p0-py+t as the data gradient's source row
-                const int hcur = p0 - 2 * kPadY + t;
-                const bool x_live = t >= kPadY && hcur >= 0 && hcur < kH;
-                const int dcur = p0 - kPadY + t;
-                const bool d_live = t < bh_eff + 2 * kPadY && dcur >= 0 && dcur < kP;
+                const int hcur = p0 - 2 * PYS + t;
+                const bool x_live = t >= PYS && hcur >= XOY && hcur < XOY + kH;
+                const int dcur = p0 - PYS + t;
+                const bool d_live = t < bh_eff + 2 * PYS && dcur >= DOY && dcur < DOY + kP;
                 const int tbase = t - sp;
-                const int own_lo = kPadY, own_hi = kPadY + bh_eff;  // owned dy rows: [own_lo, own_hi)
+                const int own_lo = PYS, own_hi = PYS + bh_eff;  // owned dy rows: [own_lo, own_hi)
                 const bool bias_pair = kDbias && sp == 1 && tbase + 1 >= own_lo && tbase < own_hi;
                 const bool do_w = wave_active && (x_live || bias_pair);
                 spio_half8 bfrag[CPW][NBLK], afrag[CPW][NPAIR];
@@ -506,7 +532,7 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                 if (!kFullUnroll || t + PF < ROWS) load_rows(xpre[pbuf], dpre[pbuf], t + PF);
 
                 // 3. the dx row finished in the previous step goes out
-                if (!kFullUnroll || t - 1 >= 2 * kPadY) store_dx_row(t - 1, (uu + 1) & 1);
+                if (!kFullUnroll || t - 1 >= 2 * PYS) store_dx_row(t - 1, (uu + 1) & 1);
 
                 // 4. rows t+1 into LDS (dy rows past the last one become zero).  The ring rows
                 //    written here are not read in this step, except for dy entries of the weight
@@ -567,7 +593,7 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                     const int slot = pmod(ph - (kR - 1), NS);
                     const int a = slot >> 1;
                     const int j = slot & 1;
-                    const bool emit = t >= 2 * kPadY && t < 2 * kPadY + bh_eff;
+                    const bool emit = t >= 2 * PYS && t < 2 * PYS + bh_eff;
                     if (wave_active && out_j == j) {
 #pragma unroll
                         for (int i = 0; i < TPW; ++i) {

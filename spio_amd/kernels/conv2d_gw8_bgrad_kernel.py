@@ -4,15 +4,17 @@ The reference launches its data-gradient and weight-gradient kernels one after
 the other (spio/functional/conv2d_gw8_function.py:119-146); both stream
 grad_output.  This family reads grad_output once and produces both gradients
 (and grad_bias when the params have a bias), which removes a quarter of the
-backward step's HBM traffic.  It exists for "same" convolutions only
-(2*padding = kernel size - 1 in both directions); `bgrad_is_supported` tells.
+backward step's HBM traffic.  The kernel computes a size-preserving convolution;
+with odd filter sizes every padding is one on a larger domain in which the input
+and the output sit centred (`bgrad_domain`), so it exists for odd filter sizes;
+`bgrad_is_supported` tells.
 
 Kernel arguments: (grad_input, grad_weight, x, grad_output, weight[, grad_bias]);
 grad_weight (and grad_bias) are accumulated into, so the caller zeroes them first.
 """
 
 from dataclasses import dataclass, replace
-from typing import Dict, List
+from typing import Dict, List, Tuple
 
 import torch
 
@@ -65,20 +67,31 @@ class Conv2dGw8BgradConfig:
 
 
 def bgrad_is_supported(params: Conv2dGw8Params) -> bool:
-    """The fused kernel needs output size = input size in both directions."""
-    return 2 * params.padding_h == params.r - 1 and 2 * params.padding_w == params.s - 1
+    """The fused kernel needs odd filter sizes.
+
+    It computes a size-preserving convolution on the domain `bgrad_domain` returns; with odd
+    filter sizes the input and the output sit centred in it, whatever the padding is.
+    """
+    return params.r % 2 == 1 and params.s % 2 == 1
+
+
+def bgrad_domain(params: Conv2dGw8Params) -> Tuple[int, int]:
+    """Rows and columns of the images the fused kernel works on: the larger of input and output."""
+    return max(params.h, params.p), max(params.w, params.q)
 
 
 def bgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig) -> Dict[str, int]:
     """Host mirror of the compile-time constants of conv2d_gw8_bgrad_mfma.hip."""
     r, s = params.r, params.s
     gb, nb, iters, ts, pf = config.groups, config.block_n, config.block_n_iters, config.split, config.prefetch
-    bh = config.block_h or params.p
+    dh, dw = bgrad_domain(params)
+    pys, pxs = (r - 1) // 2, (s - 1) // 2  # the padding of the size-preserving problem
+    bh = config.block_h or dh
     s2 = 2 * ((s + 1) // 2)
     nblk = s2 // 2
-    wpi = params.w + s - 1
+    wpi = dw + s - 1
     f = nb * wpi
-    kspan = (nb - 1) * wpi + params.q
+    kspan = (nb - 1) * wpi + dw
     kc = divup(kspan, 32)
     cpw = divup(kc, ts)
     ns = 2 * ((r + 1) // 2)
@@ -87,7 +100,7 @@ def bgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig) -> Dic
     tpw = divup(wt, ts)
     fpx = 32 * kc + s2 - 1
     gsx = fpx + ((9 - fpx % 16) + 16) % 16
-    fpd = max(params.padding_w + 32 * kc, 16 * wt + 4 * kb - 1)
+    fpd = max(pxs + 32 * kc, 16 * wt + 4 * kb - 1)
     gsd = fpd + ((9 - fpd % 16) + 16) % 16
     nrd = 4 if (params.has_bias and r == 1) else 2 * ((r + 2) // 2)
     threads = 64 * gb * ts
@@ -100,7 +113,7 @@ def bgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig) -> Dic
     publish_bytes = (gb * ts * rch * nblk * 128 + gb * (ts - 1) * nblk * 128 + gb * r * s * 64
                      + (gb * ts * 8 if params.has_bias else 0)) * 4  # fmt: skip
     lptx = divup(f * gb, threads)
-    lptd = divup(nb * params.q * gb, threads)
+    lptd = divup(nb * dw * gb, threads)
     registers = (
         4 * ((r + 1) * nblk + 1)  # weight-gradient accumulators (+ bias)
         + 4 * tpw * (ns // 2)  # data-gradient accumulators
@@ -112,9 +125,9 @@ def bgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig) -> Dic
         NBLK=nblk, KC=kc, CPW=cpw, WT=wt, TPW=tpw, THREADS=threads,
         LDS_BYTES=max(stream_bytes, filter_bytes, publish_bytes),
         LPTX=lptx, LPTD=lptd, REGISTERS=registers,
-        STEPS=bh + 3 * params.padding_h + (1 if params.has_bias and r == 1 else 0),
-        BH=bh, GBLKS=divup(params.groups, gb), PBLKS=divup(params.p, bh), NBLKS=divup(params.n, nb * iters),
-        PIXEL_EFF=(nb * params.q) / (32.0 * kc),
+        STEPS=bh + 3 * pys + (1 if params.has_bias and r == 1 else 0),
+        BH=bh, GBLKS=divup(params.groups, gb), PBLKS=divup(dh, bh), NBLKS=divup(params.n, nb * iters),
+        PIXEL_EFF=(nb * dw) / (32.0 * kc),
     )  # fmt: skip
     g["NUM_BLOCKS"] = g["GBLKS"] * g["PBLKS"] * g["NBLKS"]
     return g
@@ -127,14 +140,14 @@ def _config_is_legal(params, config) -> bool:
     return (
         config.groups * config.split <= MAX_WAVES
         and config.split <= min(g["KC"], g["WT"])
-        and 0 <= config.block_h <= params.p
+        and 0 <= config.block_h <= bgrad_domain(params)[0]
         and config.block_n * config.block_n_iters <= max(params.n, 1)
         and g["LDS_BYTES"] <= MAX_LDS_BYTES
         and g["LPTX"] <= MAX_LOADS_PER_THREAD
         and g["REGISTERS"] <= MAX_REGISTERS
         and config.prefetch >= 2
         and config.prefetch % 2 == 0
-        and config.block_n * params.c * params.h * params.w * 2 < 2**31
+        and config.block_n * params.c * max(params.h * params.w, params.p * params.q) * 2 < 2**31
     )
 
 
@@ -143,8 +156,9 @@ def _score(params, config, num_cus) -> float:
     g = bgrad_geometry(params, config)
     group_eff = params.groups / (g["GBLKS"] * config.groups)
     quant = divup(g["NUM_BLOCKS"], num_cus) * num_cus / g["NUM_BLOCKS"]
-    halo = 1.0 + (2.0 / 3.0) * (2 * params.padding_h if g["PBLKS"] > 1 else 0) / g["BH"]
-    stream_us = halo * 6.0 * params.n * params.c * params.h * params.w / 5.0e6
+    halo = 1.0 + (2.0 / 3.0) * (params.r - 1 if g["PBLKS"] > 1 else 0) / g["BH"]
+    dh, dw = bgrad_domain(params)
+    stream_us = halo * 6.0 * params.n * params.c * dh * dw / 5.0e6
     publish_us = g["NUM_BLOCKS"] * config.groups * params.r * params.s * 64.0 / (128 * 2.1e3)
     split_line = 1.0 if (config.groups * 16) % 128 == 0 or config.groups == params.groups else 1.12
     return (quant * split_line / (g["PIXEL_EFF"] ** 0.3 * group_eff)) * (1.0 + publish_us / stream_us)
@@ -161,14 +175,15 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None) -> List[Conv2dGw8Bgr
     # Rank the geometries of every row-block height separately and keep the best few of each:
     # whether whole images or row blocks win depends on the shape in ways the score does not
     # capture (contiguity of the channel block, halo re-reads, workgroups per compute unit).
-    row_choices = [0] + sorted({bh for bh in (7, 14, 28) if bh < params.p}, reverse=True)
+    dh, dw = bgrad_domain(params)
+    row_choices = [0] + sorted({bh for bh in (7, 14, 28) if bh < dh}, reverse=True)
     # images side by side: powers of two, and for rows shorter than a 32-pixel chunk of the weight
     # gradient's contraction the counts that fill the chunks clearly better (as in the
     # weight-gradient kernel's configuration space)
-    wpi = params.q + params.s - 1
+    wpi = dw + params.s - 1
 
     def chunk_fill(nb):
-        return nb * params.q / (32.0 * divup((nb - 1) * wpi + params.q, 32))
+        return nb * dw / (32.0 * divup((nb - 1) * wpi + dw, 32))
 
     image_counts = [1, 2, 4, 8]
     if wpi < 32:

@@ -58,19 +58,57 @@ def test_wgrad_sanity(params):
     run_grad_kernel_test(conv2d_gw8_wgrad_kernel_factory, params)
 
 
-# size-preserving shapes the fused backward kernel has a configuration for (7x7 needs more
-# registers than a wave has and stays with the separate kernels)
-SAME_SIZE = [p for p in SANITY if bgrad_is_supported(p) and list(conv2d_gw8_bgrad_kernel_factory.configs(p))] + [
+# shapes the fused backward kernel has a configuration for: odd filter sizes (7x7 needs more
+# registers than a wave has and stays with the separate kernels), any padding
+FUSED = [p for p in SANITY if bgrad_is_supported(p) and list(conv2d_gw8_bgrad_kernel_factory.configs(p))] + [
     Conv2dGw8Params(n=5, c=24, h=7, w=9, r=1, s=1, padding=0, has_bias=True),
     Conv2dGw8Params(n=3, c=16, h=10, w=12, r=5, s=3, padding=(2, 1), has_bias=False),
     Conv2dGw8Params(n=3, c=72, h=19, w=40, padding=1, has_bias=True),
+    # output narrower and taller than the input, and the other way round
+    Conv2dGw8Params(n=3, c=16, h=13, w=18, r=5, s=3, padding=(3, 0), has_bias=True),
+    Conv2dGw8Params(n=3, c=16, h=13, w=18, r=3, s=5, padding=(0, 4), has_bias=False),
 ]
 
 
-@pytest.mark.parametrize("params", SAME_SIZE, ids=lambda p: p.encode())
+@pytest.mark.parametrize("params", FUSED, ids=lambda p: p.encode())
 def test_bgrad_sanity(params):
-    """Fused data + weight (+ bias) gradient kernel on the size-preserving shapes."""
+    """Fused data + weight (+ bias) gradient kernel, first configurations of every shape."""
     run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params)
+
+
+def test_bgrad_when_the_image_size_changes():
+    """Paddings other than (R-1)/2: the kernel works on the larger of the two image sizes and the
+    smaller tensor sits centred in it.  Row blocks that lie partly or wholly outside the smaller
+    tensor, images side by side, split groups, a bias; the reference's sampled shapes draw their
+    padding from the same range (tests/test_conv2d_gw8.py:117-142 holds a padding-0 case)."""
+    C = Conv2dGw8BgradConfig
+    # output smaller than the input
+    params = Conv2dGw8Params(n=5, c=48, h=20, w=28, padding=0, has_bias=True)
+    run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params,
+                          configs=[C(groups=4, block_n=2, block_n_iters=1, prefetch=2, split=2),
+                                   C(groups=6, block_h=7, block_n=1, block_n_iters=2, prefetch=4, split=1),
+                                   C(groups=4, block_h=1, block_n=2, block_n_iters=1, prefetch=2, split=1)])  # fmt: skip
+    # smaller in one direction, larger in the other
+    params = Conv2dGw8Params(n=5, c=48, h=20, w=28, padding=(0, 3), has_bias=True)
+    run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params,
+                          configs=[C(groups=4, block_n=2, block_n_iters=1, prefetch=2, split=2),
+                                   C(groups=6, block_h=7, block_n=1, block_n_iters=2, prefetch=4, split=1)])  # fmt: skip
+    # output taller than the input: whole row blocks of grad_output face only padding rows of x
+    params = Conv2dGw8Params(n=5, c=48, h=20, w=28, padding=(3, 0), has_bias=False)
+    run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params,
+                          configs=[C(groups=4, block_n=2, block_n_iters=2, prefetch=4, split=1),
+                                   C(groups=6, block_h=7, block_n=1, block_n_iters=2, prefetch=4, split=1),
+                                   C(groups=4, block_h=2, block_n=1, block_n_iters=1, prefetch=2, split=1)])  # fmt: skip
+    # 5x5 filter
+    params = Conv2dGw8Params(n=3, c=16, h=13, w=18, r=5, s=5, padding=(0, 4), has_bias=True)
+    run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params,
+                          configs=[C(groups=2, block_h=5, block_n=1, block_n_iters=1, prefetch=2, split=1),
+                                   C(groups=2, block_h=3, block_n=2, block_n_iters=1, prefetch=2, split=2)])  # fmt: skip
+    # one filter row, padding rows above and below: the bias sum's extra step
+    params = Conv2dGw8Params(n=2, c=16, h=9, w=11, r=1, s=3, padding=(2, 0), has_bias=True)
+    run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params,
+                          configs=[C(groups=2, block_h=3, block_n=1, block_n_iters=1, prefetch=2, split=1),
+                                   C(groups=2, block_h=0, block_n=2, block_n_iters=1, prefetch=2, split=1)])  # fmt: skip
 
 
 def test_bgrad_explicit_configs():
@@ -113,10 +151,11 @@ def test_odd_image_counts_on_small_images():
                                    Conv2dGw8BgradConfig(groups=4, block_h=0, block_n=3, block_n_iters=2, prefetch=4, split=1)])  # fmt: skip
 
 
-def test_bgrad_is_not_offered_when_the_image_size_changes():
-    assert not bgrad_is_supported(Conv2dGw8Params(n=1, c=8, h=8, w=8, padding=0))
+def test_bgrad_is_offered_for_odd_filter_sizes():
+    assert bgrad_is_supported(Conv2dGw8Params(n=1, c=8, h=8, w=8, padding=0))
+    assert list(conv2d_gw8_bgrad_kernel_factory.configs(Conv2dGw8Params(n=1, c=8, h=8, w=8, padding=2)))
     assert not bgrad_is_supported(Conv2dGw8Params(n=1, c=8, h=8, w=8, r=4, s=1, padding=(2, 0)))
-    assert list(conv2d_gw8_bgrad_kernel_factory.configs(Conv2dGw8Params(n=1, c=8, h=8, w=8, padding=2))) == []
+    assert list(conv2d_gw8_bgrad_kernel_factory.configs(Conv2dGw8Params(n=1, c=8, h=8, w=8, r=2, s=5, padding=(1, 2)))) == []
 
 
 def test_fprop_explicit_configs():
@@ -207,7 +246,7 @@ def test_wgrad_sampled(params):
     run_grad_kernel_test(conv2d_gw8_wgrad_kernel_factory, params)
 
 
-def _sampled_same_size(seed, count=6):
+def _sampled_fused(seed, count=6):
     """Seeded draw from the reference's model-derived shapes the fused backward kernel supports."""
     import random
 
@@ -219,6 +258,6 @@ def _sampled_same_size(seed, count=6):
 
 
 @pytest.mark.slow
-@pytest.mark.parametrize("params", _sampled_same_size(seed=4), ids=lambda p: p.encode())
+@pytest.mark.parametrize("params", _sampled_fused(seed=4), ids=lambda p: p.encode())
 def test_bgrad_sampled(params):
     run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params)

@@ -127,6 +127,7 @@ def test_kernel_names_follow_the_reference_convention():
         Conv2dGw8Params(n=4, c=64, h=16, w=32, has_bias=True),
         Conv2dGw8Params(n=3, c=24, h=20, w=19, padding=(2, 0), r=4, s=1),
         Conv2dGw8Params(n=2, c=32, h=14, w=14, padding=3, r=7, s=7),
+        Conv2dGw8Params(n=3, c=24, h=20, w=19, padding=(0, 2)),
     ],
     ids=lambda p: p.encode(),
 )
@@ -135,7 +136,7 @@ def test_jit_specialisation_of_every_family(params):
     for factory, kw in ((conv2d_gw8_kernel_factory, {}), (conv2d_gw8_kernel_factory, {"igrad": True}),
                         (conv2d_gw8_wgrad_kernel_factory, {}), (conv2d_gw8_bgrad_kernel_factory, {})):  # fmt: skip
         configs = list(factory.configs(params, ATTR, **kw))
-        if not configs:  # the fused backward kernel exists for size-preserving shapes only
+        if not configs:  # the fused backward kernel exists for odd filter sizes up to 5x5 only
             assert factory is conv2d_gw8_bgrad_kernel_factory
             continue
         for cfg in {configs[0], configs[-1]}:
@@ -270,3 +271,20 @@ def test_layernorm_lane_choices():
             upl = -(-(c // 8) // lpp)
             assert lpp & (lpp - 1) == 0 and lpp * upl >= c // 8 and cfg.unroll * upl <= 8
 
+
+
+def test_fused_backward_works_on_the_larger_of_input_and_output():
+    """The fused backward kernel's grid and loads per thread follow the domain both tensors sit in:
+    the input's size where the output is smaller, the output's where it is larger."""
+    from spio_amd.kernels import Conv2dGw8BgradConfig, bgrad_is_supported
+    from spio_amd.kernels.conv2d_gw8_bgrad_kernel import bgrad_domain, bgrad_geometry
+
+    cfg = Conv2dGw8BgradConfig(groups=4, block_h=7, block_n=1)
+    same = Conv2dGw8Params(n=4, c=32, h=28, w=28, padding=1)
+    small = Conv2dGw8Params(n=4, c=32, h=28, w=28, padding=0)  # 26 x 26 output
+    large = Conv2dGw8Params(n=4, c=32, h=28, w=28, padding=(3, 1))  # 32 x 28 output
+    assert bgrad_domain(same) == bgrad_domain(small) == (28, 28) and bgrad_domain(large) == (32, 28)
+    assert bgrad_geometry(small, cfg) == bgrad_geometry(same, cfg)
+    assert bgrad_geometry(large, cfg)["PBLKS"] == 5 and bgrad_geometry(large, cfg)["STEPS"] == 7 + 3
+    assert all(bgrad_is_supported(p) for p in (same, small, large))
+    assert not bgrad_is_supported(Conv2dGw8Params(n=4, c=32, h=28, w=28, r=4, s=1, padding=(2, 0)))
