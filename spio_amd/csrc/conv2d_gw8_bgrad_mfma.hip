@@ -12,17 +12,19 @@
 // 2*|dy| + |x| + |dx| bytes through HBM; fused, dy is read once: 25 % less traffic for the
 // backward step of an HBM-bound operator, and one launch instead of two.
 //
-// Scope: odd filter sizes.  The kernel computes a "same" convolution (2*py = R-1, 2*px = S-1, so
-// P = H and Q = W): then one copy of a dy row in LDS serves both gradients, and the dx row that
-// completes at a step has the index of the x row of that step.  Any other padding of an odd
-// filter is that convolution on a larger domain, DH = max(H, P) by DW = max(W, Q), in which the
-// smaller of x and dy sits centred with zeros around it: only the global addressing knows the
-// tensors' real extents (domain rows and columns outside a tensor load zeros and store nothing),
-// and below "row", "column", py and px are the domain's.
+// Scope: every filter size and padding the operator takes.  The kernel computes a "same"
+// convolution (P = H and Q = W; padding PT rows above and PB below, PL columns left and PR right,
+// PT + PB = R-1, PL + PR = S-1): then one copy of a dy row in LDS serves both gradients, and the dx
+// row that completes at a step has the index of the x row of that step.  Any other padding is
+// that convolution on a larger domain, DH x DW, in which x and dy sit at offsets that reproduce
+// the problem's padding, with zeros around them: only the global addressing knows the tensors'
+// real extents (domain rows and columns outside a tensor load zeros and store nothing), and below
+// "row" and "column" are the domain's.
 // A workgroup owns SPIO_BH rows (of dx, and of dy for the weight gradient) of SPIO_NB images
-// side by side for SPIO_GB channel groups, repeated for SPIO_ITERS image blocks.  It streams the rows p0-py .. p0+BH-1+py of dy and of x: step t
-// stages dy row p0-py+t and x row p0-2py+t (an x row can only be multiplied once the dy rows
-// up to py below it are there).  The py halo rows of dy above and below the block feed the
+// side by side for SPIO_GB channel groups, repeated for SPIO_ITERS image blocks.  It streams the
+// rows p0-PB .. p0+BH-1+PT of dy and p0-PT .. p0+BH-1+PB of x: step t stages dy row p0-PB+t and
+// x row p0-(R-1)+t (an x row can only be multiplied once the dy rows up to PT below it are
+// there).  The halo rows of dy above and below the block feed the
 // data gradient only; the weight gradient masks them out of its dy fragments, so every dy row
 // is counted by exactly one workgroup.  With SPIO_BH = DH a workgroup owns whole images and
 // there is no halo.  Everything else is the separate kernels' design:
@@ -32,9 +34,9 @@
 //     tap pair), transposing LDS reads (see conv2d_gw8_wgrad_mfma.hip);
 //   * data gradient: A = flipped, group-transposed filter, B = dy (pixel n + tap kb is the
 //     16 bytes lane (n, kb) reads), rotating accumulator row slots (see conv2d_gw8_mfma.hip);
-//     a dy pixel (image i, column q) sits at flattened pixel i*WPI + q + px, which is both its
-//     place as a source pixel of the data gradient and, shifted by px, its place opposite x in
-//     the weight gradient;
+//     a dy pixel (image i, column q) sits at flattened pixel i*WPI + q + PR, which is both its
+//     place as a source pixel of the data gradient and, shifted by PR, its place opposite x
+//     (column c at i*WPI + c + PL) in the weight gradient;
 //   * publishing of dw (and db) as in the weight-gradient kernel: sums staged in LDS in
 //     grad_weight order, atomics of 64 consecutive floats;
 //   * global memory through buffer instructions with the hardware bounds check as predicate
@@ -73,18 +75,17 @@ using namespace spio;
 
 namespace {
 
-static_assert(kR % 2 == 1 && kS % 2 == 1, "the fused backward kernel needs odd filter sizes");
-
-// The kernel works on a size-preserving convolution of DH x DW images with the padding
-// (PYS, PXS); x (and dx) and dy sit inside that domain at the offsets (XOY, XOX) and (DOY, DOX),
-// one of each pair being 0, and count as zero around their real extent.
-constexpr int PYS = (kR - 1) / 2;
-constexpr int PXS = (kS - 1) / 2;
-constexpr int DH = kH > kP ? kH : kP;
-constexpr int DW = kW > kQ ? kW : kQ;
-constexpr int XOY = (DH - kH) / 2, XOX = (DW - kW) / 2;
-constexpr int DOY = (DH - kP) / 2, DOX = (DW - kQ) / 2;
-static_assert(DOY - XOY == PYS - kPadY && DOX - XOX == PXS - kPadX, "domain offsets");
+// The kernel works on a size-preserving convolution of DH x DW images whose padding is PT rows
+// above, PB below, PL columns left and PR right (PT + PB = R-1, PL + PR = S-1; equal halves for odd
+// filter sizes, the larger half above and left for even ones).  x (and dx) and dy sit inside that
+// domain at the offsets (XOY, XOX) and (DOY, DOX), one of each pair being 0, such that the
+// problem's own padding comes out (DOY - XOY = PT - py), and count as zero around their real extent.
+constexpr int PT = kR / 2, PB = kR - 1 - PT;
+constexpr int PL = kS / 2, PR = kS - 1 - PL;
+constexpr int DOY = PT > kPadY ? PT - kPadY : 0, XOY = PT > kPadY ? 0 : kPadY - PT;
+constexpr int DOX = PL > kPadX ? PL - kPadX : 0, XOX = PL > kPadX ? 0 : kPadX - PL;
+constexpr int DH = XOY + kH > DOY + kP ? XOY + kH : DOY + kP;
+constexpr int DW = XOX + kW > DOX + kQ ? XOX + kW : DOX + kQ;
 
 constexpr int GB = SPIO_GB;        // groups per workgroup
 constexpr int BH = SPIO_BH;        // rows per workgroup
@@ -115,7 +116,7 @@ constexpr int TPW = (WT + TS - 1) / TS;      // tiles per wave
 // ---- LDS geometry ----
 constexpr int FPX = 32 * KC + S2 - 1;  // x pixels a weight-gradient read can touch
 constexpr int GSX = FPX + ((9 - FPX % 16) + 16) % 16;  // x group stride (pixels), = 9 mod 16
-constexpr int FPD_W = PXS + 32 * KC;                   // dy pixels: weight-gradient reads
+constexpr int FPD_W = PR + 32 * KC;                    // dy pixels: weight-gradient reads
 constexpr int FPD_D = 16 * WT + 4 * KB - 1;            // dy pixels: data-gradient reads
 constexpr int FPD = FPD_W > FPD_D ? FPD_W : FPD_D;
 constexpr int GSD = FPD + ((9 - FPD % 16) + 16) % 16;  // dy group stride, = 9 mod 16
@@ -140,10 +141,10 @@ constexpr int GBLKS = (kGroups + GB - 1) / GB;
 constexpr int NBLKS = (kN + NB * ITERS - 1) / (NB * ITERS);
 constexpr int PBLKS = (DH + BH - 1) / BH;
 constexpr int NUM_BLOCKS = GBLKS * PBLKS * NBLKS;
-// steps: dy rows p0-py .. p0+BH-1+py, then py more for the last x rows.  The bias sum takes a dy
+// steps: dy rows p0-PB .. p0+BH-1+PT, then PB more for the last x rows.  The bias sum takes a dy
 // row pair one step after its first row was staged, so a one-row filter needs one more step
 // when the sum is wanted.
-constexpr int ROWS = BH + 3 * PYS + (SPIO_HAS_BIAS && kR == 1 ? 1 : 0);
+constexpr int ROWS = BH + PB + kR - 1 + (SPIO_HAS_BIAS && kR == 1 ? 1 : 0);
 
 constexpr int gcd_(int a, int b) { return b == 0 ? a : gcd_(b, a % b); }
 constexpr int LCM = NS / gcd_(NS, PF) * PF;  // lcm(NS, PF): even
@@ -243,9 +244,10 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
     const int nbk = b / (PBLKS * GBLKS);
     const int p0 = pb * BH;
     const int bh_eff = imin(BH, DH - p0);  // rows this block owns
-    // first and last row (of the domain: of x and of dy alike) the block needs
-    const int row_lo = imax(p0 - PYS, 0);
-    const int row_hi = imin(p0 + bh_eff - 1 + PYS, DH - 1);
+    // first and last row (of the domain) the block needs: of x for the weight gradient of its dy
+    // rows, of dy for its dx rows (which include the weight gradient's)
+    const int xrow_lo = p0 - PT, xrow_hi = p0 + bh_eff - 1 + PB;
+    const int drow_lo = p0 - PB, drow_hi = p0 + bh_eff - 1 + PT;
     const int gglob = cb * GB + wg;
     const bool wave_active = gglob < kGroups;
 
@@ -303,7 +305,7 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
     const int tt = lane & 3;
     const int sel = tt >> 1;
     const int xfrag_off = ((wg * GSX + 8 * kb + jr + sel) * 16) + (tt & 1) * 8;
-    const int dfrag_off = ((wg * GSD + PXS + 8 * kb + jr) * 16) + (tt & 1) * 8;
+    const int dfrag_off = ((wg * GSD + PR + 8 * kb + jr) * 16) + (tt & 1) * 8;
     // data gradient: D[m = 4*(lane/16)+i][n = lane%16]: pixel n, row slot lane/32, channels
     // 4*((lane/16)&1) + i
     const int out_j = lane >> 5;
@@ -349,7 +351,7 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                 const int g = cell % GB;
                 const int f = cell / GB;
                 const int img = f / WPI;
-                const int col = f % WPI - PXS - XOX;  // column of x
+                const int col = f % WPI - PL - XOX;  // column of x
                 x_lds[l] = g * GSX + f;
                 if (col >= 0 && col < kW && cb * GB + g < kGroups)
                     x_voff[l] = (unsigned)(((img * kH * kW + col) * kGroups + cb * GB + g) * 16);
@@ -370,7 +372,7 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                 const int g = cell % GB;
                 const int q = (cell / GB) % DW;
                 const int img = cell / (GB * DW);
-                d_lds[l] = g * GSD + img * WPI + q + PXS;
+                d_lds[l] = g * GSD + img * WPI + q + PR;
                 o_lds[l] = (img * WPI + q) * OSTRIDE + g * 16;
                 const int qd = q - DOX;  // column of dy
                 const int wx = q - XOX;  // column of dx
@@ -381,12 +383,12 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
             }
         }
 
-        // Rows `t` of x (domain row p0-2py+t) and of dy (p0-py+t) for every cell of the thread.
+        // Rows `t` of x (domain row p0-(R-1)+t) and of dy (p0-PB+t) for every cell of the thread.
         // Rows the block does not need, and domain rows outside the tensor, read through the empty
         // descriptor (zeros, no traffic).
         auto load_rows = [&](spio_uint4(&xr)[LPTX], spio_uint4(&dr)[LPTD], int t) {
-            const int h = p0 - 2 * PYS + t;
-            const rsrc_t rx = (h >= row_lo && h <= row_hi && h >= XOY && h < XOY + kH) ? rs_x : rs_none;
+            const int h = p0 - (kR - 1) + t;
+            const rsrc_t rx = (h >= xrow_lo && h <= xrow_hi && h >= XOY && h < XOY + kH) ? rs_x : rs_none;
             const int sx = __builtin_amdgcn_readfirstlane(imin(imax(h - XOY, 0), kH - 1) * X_ROW_BYTES);
             const bool xhalo = h < p0 || h >= p0 + bh_eff;
 #pragma unroll
@@ -396,8 +398,8 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                                                   : __builtin_amdgcn_raw_buffer_load_b128(rx, (int)x_voff[l], sx, AUX_NT);
                 xr[l] = v.u;
             }
-            const int pr = p0 - PYS + t;
-            const rsrc_t rd = (pr >= row_lo && pr <= row_hi && pr >= DOY && pr < DOY + kP) ? rs_dy : rs_none;
+            const int pr = p0 - PB + t;
+            const rsrc_t rd = (pr >= drow_lo && pr <= drow_hi && pr >= DOY && pr < DOY + kP) ? rs_dy : rs_none;
             const int sd = __builtin_amdgcn_readfirstlane(imin(imax(pr - DOY, 0), kP - 1) * D_ROW_BYTES);
             const bool dhalo = pr < p0 || pr >= p0 + bh_eff;
 #pragma unroll
@@ -432,13 +434,13 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
 #pragma unroll
             for (int a = 0; a < NACC; ++a) dacc[i][a] = spio_float4{0.f, 0.f, 0.f, 0.f};
 
-        // Coalesced store of the dx row staged at step `ts` (domain row p0 - 2py + ts), one step
+        // Coalesced store of the dx row staged at step `ts` (domain row p0 - (R-1) + ts), one step
         // later.  Steps that finish no row of the block, or a domain row outside dx, store through
         // the empty descriptor: the
         // instructions are issued all the same and the hardware drops them.
         auto store_dx_row = [&](int ts, int obuf) {
-            const int h = p0 - 2 * PYS + ts;
-            const bool real = ts >= 2 * PYS && ts < 2 * PYS + bh_eff && h >= XOY && h < XOY + kH;
+            const int h = p0 - (kR - 1) + ts;
+            const bool real = ts >= kR - 1 && ts < kR - 1 + bh_eff && h >= XOY && h < XOY + kH;
             const rsrc_t rs = real ? rs_dx : rs_none;
             // The row offset is added to the per-lane offset; the scalar-offset operand stays the
             // constant 0.  A 16-byte buffer store reads its data registers for a few cycles after
@@ -465,15 +467,15 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                 const int ph = uu % NS;                  // data-gradient phase: t mod NS
                 const int obuf = uu & 1;
 
-                // 1. fragment reads: x row p0-2py+t, the dy row pairs it meets (dy rows are named
-                //    by the step that staged them: row p0-py+tau at step tau; the block owns
-                //    tau in [py, py+bh_eff)), and dy row p0-py+t as the data gradient's source row
-                const int hcur = p0 - 2 * PYS + t;
-                const bool x_live = t >= PYS && hcur >= XOY && hcur < XOY + kH;
-                const int dcur = p0 - PYS + t;
-                const bool d_live = t < bh_eff + 2 * PYS && dcur >= DOY && dcur < DOY + kP;
+                // 1. fragment reads: x row p0-(R-1)+t, the dy row pairs it meets (dy rows are named
+                //    by the step that staged them: row p0-PB+tau at step tau; the block owns
+                //    tau in [PB, PB+bh_eff)), and dy row p0-PB+t as the data gradient's source row
+                const int hcur = p0 - (kR - 1) + t;
+                const bool x_live = t >= PB && hcur >= XOY && hcur < XOY + kH;
+                const int dcur = p0 - PB + t;
+                const bool d_live = t < bh_eff + kR - 1 && dcur >= DOY && dcur < DOY + kP;
                 const int tbase = t - sp;
-                const int own_lo = PYS, own_hi = PYS + bh_eff;  // owned dy rows: [own_lo, own_hi)
+                const int own_lo = PB, own_hi = PB + bh_eff;  // owned dy rows: [own_lo, own_hi)
                 const bool bias_pair = kDbias && sp == 1 && tbase + 1 >= own_lo && tbase < own_hi;
                 const bool do_w = wave_active && (x_live || bias_pair);
                 spio_half8 bfrag[CPW][NBLK], afrag[CPW][NPAIR];
@@ -532,7 +534,7 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                 if (!kFullUnroll || t + PF < ROWS) load_rows(xpre[pbuf], dpre[pbuf], t + PF);
 
                 // 3. the dx row finished in the previous step goes out
-                if (!kFullUnroll || t - 1 >= 2 * PYS) store_dx_row(t - 1, (uu + 1) & 1);
+                if (!kFullUnroll || t - 1 >= kR - 1) store_dx_row(t - 1, (uu + 1) & 1);
 
                 // 4. rows t+1 into LDS (dy rows past the last one become zero).  The ring rows
                 //    written here are not read in this step, except for dy entries of the weight
@@ -587,13 +589,13 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                     }
                 }
 
-                // 6. the dx row that received its last tap (row p0-2py+t): stage it if the block
+                // 6. the dx row that received its last tap (row p0-(R-1)+t): stage it if the block
                 //    owns it, reset its slot
                 {
                     const int slot = pmod(ph - (kR - 1), NS);
                     const int a = slot >> 1;
                     const int j = slot & 1;
-                    const bool emit = t >= 2 * PYS && t < 2 * PYS + bh_eff;
+                    const bool emit = t >= kR - 1 && t < kR - 1 + bh_eff;
                     if (wave_active && out_j == j) {
 #pragma unroll
                         for (int i = 0; i < TPW; ++i) {

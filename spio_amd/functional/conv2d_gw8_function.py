@@ -13,10 +13,10 @@ One deliberate difference: the fake implementation of the backward op reports
 grad_weight as fp32, which is what the real op returns (the reference's fake
 says fp16, :164).
 
-When grad_input and grad_weight are both wanted and the filter sizes are
-odd, the backward op can run one fused kernel that reads grad_output
-once instead of the reference's two launches (:119-146).  SPIO_FUSED_BACKWARD=0
-never fuses, =1 fuses whenever the shape allows, anything else (default) fuses
+When grad_input and grad_weight are both wanted, the backward op can run one
+fused kernel that reads grad_output once instead of the reference's two
+launches (:119-146).  SPIO_FUSED_BACKWARD=0 never fuses, =1 fuses whenever the
+shape has a fused configuration, anything else (default) fuses
 when the recorded kernel times say it is faster, or, without records, when the
 fused kernel has enough workgroups to fill the device.
 """

@@ -5,9 +5,8 @@ the other (spio/functional/conv2d_gw8_function.py:119-146); both stream
 grad_output.  This family reads grad_output once and produces both gradients
 (and grad_bias when the params have a bias), which removes a quarter of the
 backward step's HBM traffic.  The kernel computes a size-preserving convolution;
-with odd filter sizes every padding is one on a larger domain in which the input
-and the output sit centred (`bgrad_domain`), so it exists for odd filter sizes;
-`bgrad_is_supported` tells.
+every other padding is one on a larger domain in which the input and the output
+sit at fitting offsets (`bgrad_domain`).
 
 Kernel arguments: (grad_input, grad_weight, x, grad_output, weight[, grad_bias]);
 grad_weight (and grad_bias) are accumulated into, so the caller zeroes them first.
@@ -67,17 +66,29 @@ class Conv2dGw8BgradConfig:
 
 
 def bgrad_is_supported(params: Conv2dGw8Params) -> bool:
-    """The fused kernel needs odd filter sizes.
+    """The fused kernel takes every shape the operator takes.
 
-    It computes a size-preserving convolution on the domain `bgrad_domain` returns; with odd
-    filter sizes the input and the output sit centred in it, whatever the padding is.
+    It computes a size-preserving convolution on the domain `bgrad_domain` returns, in which the
+    input and the output sit at offsets that reproduce the problem's padding.  Whether a shape
+    has a legal configuration is a separate question (large filters run out of registers).
     """
-    return params.r % 2 == 1 and params.s % 2 == 1
+    return params.r >= 1 and params.s >= 1
 
 
 def bgrad_domain(params: Conv2dGw8Params) -> Tuple[int, int]:
-    """Rows and columns of the images the fused kernel works on: the larger of input and output."""
-    return max(params.h, params.p), max(params.w, params.q)
+    """Rows and columns of the images the fused kernel works on.
+
+    The domain's own padding is r // 2 rows above (s // 2 columns left) and the rest of r - 1
+    (s - 1) below (right); the input starts max(padding - r // 2, 0) rows into the domain, the
+    output max(r // 2 - padding, 0), and the domain ends where the later of the two ends.
+    """
+
+    def extent(size, out_size, filt, padding):
+        shift = filt // 2 - padding
+        return max(max(-shift, 0) + size, max(shift, 0) + out_size)
+
+    return (extent(params.h, params.p, params.r, params.padding_h),
+            extent(params.w, params.q, params.s, params.padding_w))  # fmt: skip
 
 
 def bgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig) -> Dict[str, int]:
@@ -85,7 +96,7 @@ def bgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig) -> Dic
     r, s = params.r, params.s
     gb, nb, iters, ts, pf = config.groups, config.block_n, config.block_n_iters, config.split, config.prefetch
     dh, dw = bgrad_domain(params)
-    pys, pxs = (r - 1) // 2, (s - 1) // 2  # the padding of the size-preserving problem
+    pb, pr = r - 1 - r // 2, s - 1 - s // 2  # the domain's padding below and right
     bh = config.block_h or dh
     s2 = 2 * ((s + 1) // 2)
     nblk = s2 // 2
@@ -100,7 +111,7 @@ def bgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig) -> Dic
     tpw = divup(wt, ts)
     fpx = 32 * kc + s2 - 1
     gsx = fpx + ((9 - fpx % 16) + 16) % 16
-    fpd = max(pxs + 32 * kc, 16 * wt + 4 * kb - 1)
+    fpd = max(pr + 32 * kc, 16 * wt + 4 * kb - 1)
     gsd = fpd + ((9 - fpd % 16) + 16) % 16
     nrd = 4 if (params.has_bias and r == 1) else 2 * ((r + 2) // 2)
     threads = 64 * gb * ts
@@ -125,7 +136,7 @@ def bgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig) -> Dic
         NBLK=nblk, KC=kc, CPW=cpw, WT=wt, TPW=tpw, THREADS=threads,
         LDS_BYTES=max(stream_bytes, filter_bytes, publish_bytes),
         LPTX=lptx, LPTD=lptd, REGISTERS=registers,
-        STEPS=bh + 3 * pys + (1 if params.has_bias and r == 1 else 0),
+        STEPS=bh + pb + r - 1 + (1 if params.has_bias and r == 1 else 0),
         BH=bh, GBLKS=divup(params.groups, gb), PBLKS=divup(dh, bh), NBLKS=divup(params.n, nb * iters),
         PIXEL_EFF=(nb * dw) / (32.0 * kc),
     )  # fmt: skip

@@ -122,7 +122,9 @@ def test_backward_op_fused_and_separate_kernels_agree_with_the_oracle(monkeypatc
               Conv2dGw8Params(n=2, c=16, h=9, w=9, r=5, s=5, padding=2, has_bias=False),
               # output smaller and larger than the input
               Conv2dGw8Params(n=3, c=40, h=12, w=20, padding=0, has_bias=True),
-              Conv2dGw8Params(n=2, c=16, h=9, w=9, r=5, s=3, padding=(3, 2), has_bias=True)):  # fmt: skip
+              Conv2dGw8Params(n=2, c=16, h=9, w=9, r=5, s=3, padding=(3, 2), has_bias=True),
+              # even filter sizes (the reference's regression shape, tests/test_conv2d_gw8.py:176-180)
+              Conv2dGw8Params(n=4, c=128, h=32, w=32, r=4, s=1, padding=(2, 0), has_bias=True)):  # fmt: skip
         x, w, b, dy = oracle.make_args(p.n, p.c, p.h, p.w, p.r, p.s, p.padding_h, p.padding_w, p.has_bias, 3)
         dx_e, dw_e, db_e = oracle.grads_torch(x, w, b, dy, p.padding_h, p.padding_w)
         dx, dw, db = torch.ops.spio.conv2d_gw8_backward(
@@ -145,8 +147,9 @@ def test_fused_backward_choice(monkeypatch):
     monkeypatch.setenv("SPIO_FUSED_BACKWARD", "1")
     assert fused_backward_kernel(same, dev) is not None
     assert fused_backward_kernel(Conv2dGw8Params(n=2, c=16, h=8, w=8, padding=0), dev) is not None
-    # even filter sizes stay with the separate kernels
-    assert fused_backward_kernel(Conv2dGw8Params(n=2, c=16, h=8, w=8, r=4, s=1, padding=(2, 0)), dev) is None
+    assert fused_backward_kernel(Conv2dGw8Params(n=2, c=16, h=8, w=8, r=4, s=1, padding=(2, 0)), dev) is not None
+    # 7x7 has no fused configuration: the separate kernels
+    assert fused_backward_kernel(Conv2dGw8Params(n=2, c=16, h=8, w=8, r=7, s=7, padding=3), dev) is None
     # no recorded times for this shape and far fewer workgroups than compute units: separate kernels
     monkeypatch.setenv("SPIO_FUSED_BACKWARD", "auto")
     assert fused_backward_kernel(same, dev) is None

@@ -58,8 +58,8 @@ def test_wgrad_sanity(params):
     run_grad_kernel_test(conv2d_gw8_wgrad_kernel_factory, params)
 
 
-# shapes the fused backward kernel has a configuration for: odd filter sizes (7x7 needs more
-# registers than a wave has and stays with the separate kernels), any padding
+# shapes the fused backward kernel has a configuration for: any padding, odd and even filter
+# sizes (7x7 needs more registers than a wave has and stays with the separate kernels)
 FUSED = [p for p in SANITY if bgrad_is_supported(p) and list(conv2d_gw8_bgrad_kernel_factory.configs(p))] + [
     Conv2dGw8Params(n=5, c=24, h=7, w=9, r=1, s=1, padding=0, has_bias=True),
     Conv2dGw8Params(n=3, c=16, h=10, w=12, r=5, s=3, padding=(2, 1), has_bias=False),
@@ -77,10 +77,11 @@ def test_bgrad_sanity(params):
 
 
 def test_bgrad_when_the_image_size_changes():
-    """Paddings other than (R-1)/2: the kernel works on the larger of the two image sizes and the
-    smaller tensor sits centred in it.  Row blocks that lie partly or wholly outside the smaller
-    tensor, images side by side, split groups, a bias; the reference's sampled shapes draw their
-    padding from the same range (tests/test_conv2d_gw8.py:117-142 holds a padding-0 case)."""
+    """Paddings other than (R-1)/2, and even filter sizes: the kernel works on a domain that holds
+    both tensors at offsets that reproduce the padding.  Row blocks that lie partly or wholly
+    outside the smaller tensor, images side by side, split groups, a bias; the reference's sampled
+    shapes draw their padding from the same range (tests/test_conv2d_gw8.py:80-85) and its
+    regression cases hold r=4, s=1, padding=(2, 0) (tests/test_conv2d_gw8.py:176-180)."""
     C = Conv2dGw8BgradConfig
     # output smaller than the input
     params = Conv2dGw8Params(n=5, c=48, h=20, w=28, padding=0, has_bias=True)
@@ -104,6 +105,23 @@ def test_bgrad_when_the_image_size_changes():
     run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params,
                           configs=[C(groups=2, block_h=5, block_n=1, block_n_iters=1, prefetch=2, split=1),
                                    C(groups=2, block_h=3, block_n=2, block_n_iters=1, prefetch=2, split=2)])  # fmt: skip
+    # even filter sizes: the output is one row or column larger or smaller than the input
+    params = Conv2dGw8Params(n=4, c=128, h=32, w=32, r=4, s=1, padding=(2, 0), has_bias=True)
+    run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params,
+                          configs=[C(groups=8, block_h=7, block_n=1, block_n_iters=1, prefetch=2, split=1),
+                                   C(groups=4, block_h=0, block_n=2, block_n_iters=2, prefetch=4, split=1)])  # fmt: skip
+    params = Conv2dGw8Params(n=5, c=32, h=17, w=21, r=4, s=4, padding=(0, 3), has_bias=True)
+    run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params,
+                          configs=[C(groups=4, block_h=5, block_n=1, block_n_iters=1, prefetch=2, split=1),
+                                   C(groups=2, block_h=0, block_n=2, block_n_iters=2, prefetch=4, split=2),
+                                   C(groups=4, block_h=1, block_n=1, block_n_iters=1, prefetch=2, split=1)])  # fmt: skip
+    params = Conv2dGw8Params(n=5, c=32, h=17, w=21, r=2, s=2, padding=(1, 0), has_bias=False)
+    run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params,
+                          configs=[C(groups=4, block_h=5, block_n=1, block_n_iters=1, prefetch=2, split=1),
+                                   C(groups=2, block_h=0, block_n=2, block_n_iters=2, prefetch=4, split=2)])  # fmt: skip
+    params = Conv2dGw8Params(n=5, c=32, h=17, w=21, r=3, s=2, padding=(1, 1), has_bias=True)
+    run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params,
+                          configs=[C(groups=4, block_h=7, block_n=2, block_n_iters=1, prefetch=2, split=1)])  # fmt: skip
     # one filter row, padding rows above and below: the bias sum's extra step
     params = Conv2dGw8Params(n=2, c=16, h=9, w=11, r=1, s=3, padding=(2, 0), has_bias=True)
     run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params,
@@ -151,11 +169,13 @@ def test_odd_image_counts_on_small_images():
                                    Conv2dGw8BgradConfig(groups=4, block_h=0, block_n=3, block_n_iters=2, prefetch=4, split=1)])  # fmt: skip
 
 
-def test_bgrad_is_offered_for_odd_filter_sizes():
-    assert bgrad_is_supported(Conv2dGw8Params(n=1, c=8, h=8, w=8, padding=0))
-    assert list(conv2d_gw8_bgrad_kernel_factory.configs(Conv2dGw8Params(n=1, c=8, h=8, w=8, padding=2)))
-    assert not bgrad_is_supported(Conv2dGw8Params(n=1, c=8, h=8, w=8, r=4, s=1, padding=(2, 0)))
-    assert list(conv2d_gw8_bgrad_kernel_factory.configs(Conv2dGw8Params(n=1, c=8, h=8, w=8, r=2, s=5, padding=(1, 2)))) == []
+def test_bgrad_is_offered_for_every_padding_and_filter_parity():
+    for params in (Conv2dGw8Params(n=1, c=8, h=8, w=8, padding=0), Conv2dGw8Params(n=1, c=8, h=8, w=8, padding=2),
+                   Conv2dGw8Params(n=1, c=8, h=8, w=8, r=4, s=1, padding=(2, 0)),
+                   Conv2dGw8Params(n=1, c=8, h=8, w=8, r=2, s=5, padding=(1, 2))):  # fmt: skip
+        assert bgrad_is_supported(params) and list(conv2d_gw8_bgrad_kernel_factory.configs(params))
+    # 7x7: no configuration fits the registers
+    assert list(conv2d_gw8_bgrad_kernel_factory.configs(Conv2dGw8Params(n=2, c=32, h=14, w=14, r=7, s=7, padding=3))) == []
 
 
 def test_fprop_explicit_configs():

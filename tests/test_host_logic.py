@@ -136,7 +136,7 @@ def test_jit_specialisation_of_every_family(params):
     for factory, kw in ((conv2d_gw8_kernel_factory, {}), (conv2d_gw8_kernel_factory, {"igrad": True}),
                         (conv2d_gw8_wgrad_kernel_factory, {}), (conv2d_gw8_bgrad_kernel_factory, {})):  # fmt: skip
         configs = list(factory.configs(params, ATTR, **kw))
-        if not configs:  # the fused backward kernel exists for odd filter sizes up to 5x5 only
+        if not configs:  # the fused backward kernel has no configuration for 7x7 (registers)
             assert factory is conv2d_gw8_bgrad_kernel_factory
             continue
         for cfg in {configs[0], configs[-1]}:
@@ -275,7 +275,8 @@ def test_layernorm_lane_choices():
 
 def test_fused_backward_works_on_the_larger_of_input_and_output():
     """The fused backward kernel's grid and loads per thread follow the domain both tensors sit in:
-    the input's size where the output is smaller, the output's where it is larger."""
+    the input's size where the output is smaller, the output's where it is larger; with an even
+    filter size the two are offset by half a pixel and the domain holds both."""
     from spio_amd.kernels import Conv2dGw8BgradConfig, bgrad_is_supported
     from spio_amd.kernels.conv2d_gw8_bgrad_kernel import bgrad_domain, bgrad_geometry
 
@@ -286,5 +287,7 @@ def test_fused_backward_works_on_the_larger_of_input_and_output():
     assert bgrad_domain(same) == bgrad_domain(small) == (28, 28) and bgrad_domain(large) == (32, 28)
     assert bgrad_geometry(small, cfg) == bgrad_geometry(same, cfg)
     assert bgrad_geometry(large, cfg)["PBLKS"] == 5 and bgrad_geometry(large, cfg)["STEPS"] == 7 + 3
-    assert all(bgrad_is_supported(p) for p in (same, small, large))
-    assert not bgrad_is_supported(Conv2dGw8Params(n=4, c=32, h=28, w=28, r=4, s=1, padding=(2, 0)))
+    even = Conv2dGw8Params(n=4, c=32, h=28, w=28, r=4, s=1, padding=(2, 0))  # 29 x 28 output
+    assert bgrad_domain(even) == (29, 28) and bgrad_geometry(even, cfg)["STEPS"] == 7 + 1 + 3
+    assert bgrad_domain(Conv2dGw8Params(n=4, c=32, h=28, w=28, r=4, s=4, padding=(0, 3))) == (28, 31)
+    assert all(bgrad_is_supported(p) for p in (same, small, large, even))
