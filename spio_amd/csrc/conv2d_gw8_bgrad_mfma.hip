@@ -255,46 +255,24 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
     // A[m = dx channel ch][jj] = w[8g+jj][R-1-r][S-1-s][ch].  The workgroup copies its groups'
     // filters to LDS as they lie in memory and every wave reads its fragments with the
     // transposing LDS read (same scheme as the data-gradient mode of conv2d_gw8_mfma.hip).
-    spio_half8 wfrag[NS][KB];
+    // The filter loads are issued here, the loads of the first rows right behind them, and only
+    // then does anything wait: the fragments are built while the rows are on their way.
+    constexpr int FLT = (FILTER_UNITS + THREADS - 1) / THREADS;
+    spio_uint4 fpre[FLT];
     {
-        for (int i = tid; i < FILTER_UNITS; i += THREADS) {
-            const int g = i / (8 * kR * kS);
-            const int rem = i % (8 * kR * kS);
-            spio_uint4 v = spio_uint4{0u, 0u, 0u, 0u};
-            if (cb * GB + g < kGroups)
-                v = reinterpret_cast<const spio_uint4*>(weights)[(long long)(cb * GB + g) * (8 * kR * kS) + rem];
-            lds[i] = v;
-        }
-        block_sync();
-        const int kbl = lane >> 4;
-        const int jr = (lane & 15) >> 2;
-        const int t4 = lane & 3;
-        const int src_slot = t4 >> 1;
-        const int my_slot = (lane & 15) >> 3;
-        typedef spio_short4 __attribute__((address_space(3))) * lds_ptr;
+        const int valid_groups = imin(GB, kGroups - cb * GB);
+        const rsrc_t rs_w = make_rsrc(reinterpret_cast<const unsigned char*>(weights) +
+                                          (long long)cb * GB * (8 * kR * kS * 16),
+                                      valid_groups * (8 * kR * kS * 16));
 #pragma unroll
-        for (int d = 0; d < NS; ++d) {
-#pragma unroll
-            for (int u = 0; u < KB; ++u) {
-                const int s = 4 * u + kbl;
-                const int r_src = (d - src_slot + NS) % NS;
-                const int r_mine = (d - my_slot + NS) % NS;
-                const int rr = r_src < kR ? kR - 1 - r_src : 0;  // dead taps: any valid address
-                const int ss = s < kS ? kS - 1 - s : 0;
-                const unsigned char* base = reinterpret_cast<const unsigned char*>(lds) +
-                                            ((((wg * 8 + jr) * kR + rr) * kS + ss) * 16) + (t4 & 1) * 8;
-                union {
-                    spio_short4 q[2];
-                    spio_half8 h;
-                } v;
-                v.q[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)base);
-                v.q[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(base + 4 * kR * kS * 16));
-                if (!(wave_active && r_mine < kR && s < kS)) v.h = spio_half8{0, 0, 0, 0, 0, 0, 0, 0};
-                wfrag[d][u] = v.h;
-            }
+        for (int l = 0; l < FLT; ++l) {
+            Pack16 v;  // units past the workgroup's groups lie beyond the descriptor: zeros
+            v.i = __builtin_amdgcn_raw_buffer_load_b128(rs_w, (tid + THREADS * l) * 16, 0, 0);
+            fpre[l] = v.u;
         }
-        block_sync();  // everyone has its fragments before the rings are zero-filled
     }
+    __builtin_amdgcn_sched_barrier(0);  // keep the filter loads ahead of the row loads
+    spio_half8 wfrag[NS][KB];
 
     // ---- lane roles ----
     // weight gradient (transposing reads): block kb = lane/16 covers pixels 8*kb..8*kb+7, source
@@ -417,8 +395,42 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
         for (int t = 0; t < PF; ++t) load_rows(xpre[t], dpre[t], t);
         __builtin_amdgcn_sched_barrier(0);  // the first loads are on their way before anything waits
         if (it == 0) {
-            // zero both rings once, while the first loads are in flight: the slack cells behind
-            // each group's pixels are never written
+            // while the first loads are in flight: the filter fragments, through the LDS block
+            // the rings will use ...
+#pragma unroll
+            for (int l = 0; l < FLT; ++l)
+                if (tid + THREADS * l < FILTER_UNITS) lds[tid + THREADS * l] = fpre[l];
+            block_sync();
+            const int fkb = lane >> 4;
+            const int fjr = (lane & 15) >> 2;
+            const int ft4 = lane & 3;
+            const int src_slot = ft4 >> 1;
+            const int my_slot = (lane & 15) >> 3;
+            typedef spio_short4 __attribute__((address_space(3))) * lds_ptr;
+#pragma unroll
+            for (int d = 0; d < NS; ++d) {
+#pragma unroll
+                for (int u = 0; u < KB; ++u) {
+                    const int s = 4 * u + fkb;
+                    const int r_src = (d - src_slot + NS) % NS;
+                    const int r_mine = (d - my_slot + NS) % NS;
+                    const int rr = r_src < kR ? kR - 1 - r_src : 0;  // dead taps: any valid address
+                    const int ss = s < kS ? kS - 1 - s : 0;
+                    const unsigned char* base = reinterpret_cast<const unsigned char*>(lds) +
+                                                ((((wg * 8 + fjr) * kR + rr) * kS + ss) * 16) + (ft4 & 1) * 8;
+                    union {
+                        spio_short4 q[2];
+                        spio_half8 h;
+                    } v;
+                    v.q[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)base);
+                    v.q[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(base + 4 * kR * kS * 16));
+                    if (!(wave_active && r_mine < kR && s < kS)) v.h = spio_half8{0, 0, 0, 0, 0, 0, 0, 0};
+                    wfrag[d][u] = v.h;
+                }
+            }
+            block_sync();  // everyone has its fragments before the rings are zero-filled
+            // ... and both rings zeroed once: the slack cells behind each group's pixels are
+            // never written
             for (int i = tid; i < RING_UNITS; i += THREADS) lds[i] = zero4;
         }
         block_sync();  // rings zeroed / previous image block finished
