@@ -192,7 +192,7 @@ def main(argv=None):
     ap.add_argument("shapes", nargs="*", help="shapes in Conv2dGw8Params.encode() form")
     ap.add_argument("--shapes", dest="preset", choices=["bench", "batch-sweep", "network", "all"])
     ap.add_argument("--directions", default="fprop,dgrad,wgrad,bgrad",
-                    help="bgrad = the fused data+weight gradient kernel (size-preserving shapes only)")
+                    help="bgrad = the fused data+weight gradient kernel")
     ap.add_argument("--iters", type=int, default=30)
     ap.add_argument("--package", action="store_true", help="write into spio_amd/kernels/tuned/")
     args = ap.parse_args(argv)
