@@ -12,6 +12,9 @@ Workloads (--workload):
              times, so the rates are HBM rates.
   cfg4       forward (and backward) at C=64 56x56 3x3 for batch sizes 1..512.
   cfg5       inference of a ConvNeXt-Tiny-shaped network with gw8 convolutions at batch 128.
+The default run (target) also carries a `configs` block: compact measurements of cfg1, cfg2, cfg3
+(per-kernel us, fraction of the HBM roofline, counter traffic), the cfg4 batch sweep and cfg5 (the
+four convolution and LayerNorm shapes and the network's ms per iteration); --no-configs leaves it out.
 
 The single JSON line printed at the end reports
   value      effective GB/s of the whole step = the algorithmic bytes the launched kernels move
@@ -20,8 +23,9 @@ The single JSON line printed at the end reports
              byte count (scripts/plot_kernel_bench.py:430-435),
   kernels    per-kernel us (median and min over repeated event-timed blocks), effective GB/s and
              fraction of the 8 TB/s roofline,
-  roofline   the same for the kernel that takes the most time, with the HBM traffic measured by
-             rocprofv3 counters when a summary for this workload is in profiles/,
+  roofline   the same for the kernel that takes the most time, with the HBM traffic and the MFMA
+             utilisation measured by rocprofv3 counters when a summary for this workload is in
+             profiles/ (`traffic_stale` / `mfma_util_stale`: the kernel source has changed since),
   copy_ceiling  the best of a few tuned streaming copies of the same volume (what HBM gives a
              read-X/write-X kernel on this device), and the plain copy beside it,
   torch_gpu_conv2d  torch's own grouped conv2d (MIOpen) on the same GPU and shapes,
@@ -45,6 +49,8 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
+# the run-time compiler's thread pool: the benchmark compiles some sixty kernels (read at import)
+os.environ.setdefault("SPIO_WORKERS", str(max(4, min(16, (os.cpu_count() or 4)))))
 
 HBM_PEAK_GBS = 8000.0
 CACHE_BYTES = 256 * 1024 * 1024
@@ -76,23 +82,44 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-torch-gpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-batch", type=int, default=32)
+    ap.add_argument("--no-configs", action="store_true",
+                    help="default workload only: leave out the compact cfg1-cfg5 block")
     return ap.parse_args()
 
 
 # ------------------------------------------------------------------ helpers
 
 
-def measured_traffic(workload, kernel):
-    """HBM bytes per launch from the rocprofv3 counter summaries in profiles/, or None.
+def source_digest(source_file):
+    """Short hash of a kernel source and the header it includes: what a counter figure in
+    profiles/ was measured with."""
+    import hashlib
 
-    The summaries carry lines `traffic_bytes <workload> <kernel> <bytes>` (FETCH_SIZE + WRITE_SIZE
-    per dispatch, each scaled by what the same counter reads for the plain copy kernel)."""
+    h = hashlib.sha256()
+    for name in (source_file, "spio_conv_common.h"):
+        try:
+            with open(os.path.join(ROOT, "spio_amd", "csrc", name), "rb") as f:
+                h.update(f.read())
+        except OSError:
+            return None
+    return h.hexdigest()[:12]
+
+
+def profile_figure(kind, workload, kernel, source_file=None):
+    """A per-launch figure from the rocprofv3 counter summaries in profiles/: (value, stale).
+
+    The summaries carry lines `<kind> <workload> <kernel> <value> [<source file>:<digest>]` with
+    kind `traffic_bytes` (FETCH_SIZE + WRITE_SIZE per dispatch, each scaled by what the same
+    counter reads for the plain copy kernel) or `mfma_util` (per cent of the cycles in which the
+    matrix pipes were busy, the profiler's MfmaUtil).  `stale` is True when the line names the
+    digest of the kernel source it was measured with and today's source differs, None when it
+    names none.  (None, None) without a summary."""
     pdir = os.path.join(ROOT, "profiles")
     try:
         names = sorted(os.listdir(pdir))
     except OSError:
-        return None
-    pat = re.compile(rf"traffic_bytes\s+{re.escape(workload)}\s+{re.escape(kernel)}\s+(\d+)")
+        return None, None
+    pat = re.compile(rf"{kind}\s+{re.escape(workload)}\s+{re.escape(kernel)}\s+([0-9.]+)(?:\s+(\S+):([0-9a-f]+))?")
     for name in names:
         try:
             with open(os.path.join(pdir, name), "r", encoding="utf-8") as f:
@@ -100,8 +127,24 @@ def measured_traffic(workload, kernel):
         except OSError:
             continue
         if m:
-            return int(m.group(1))
-    return None
+            value = float(m.group(1)) if kind == "mfma_util" else int(float(m.group(1)))
+            stale = None
+            if m.group(3):
+                stale = source_digest(m.group(2)) != m.group(3)
+            return value, stale
+    return None, None
+
+
+def attach_profile_figures(entry, workload, name):
+    """Adds traffic / mfma_util (and their stale flags) from profiles/ to a kernel entry."""
+    entry["traffic"], stale = profile_figure("traffic_bytes", workload, name)
+    if stale is not None:
+        entry["traffic_stale"] = stale
+    util, ustale = profile_figure("mfma_util", workload, name)
+    if util is not None:
+        entry["mfma_util"] = round(util / 100.0, 4)
+        if ustale is not None:
+            entry["mfma_util_stale"] = ustale
 
 
 def rotation_sets(set_bytes):
@@ -121,20 +164,20 @@ def timed_blocks(run_block, min_seconds=MIN_TIMED_SECONDS, max_blocks=400):
     return times
 
 
-def time_kernel(kernel, arg_sets, iters):
+def time_kernel(kernel, arg_sets, iters, min_seconds=MIN_TIMED_SECONDS):
     """Median and min microseconds per call over repeated event-timed blocks of `iters` launches."""
     kernel.time(arg_sets, warmup=10, iters=iters)
     per_call = []
     total = 0.0
-    while (total < MIN_TIMED_SECONDS or len(per_call) < 3) and len(per_call) < 400:
+    while (total < min_seconds or len(per_call) < 3) and len(per_call) < 400:
         ms = kernel.time(arg_sets, warmup=0, iters=iters)
         per_call.append(ms * 1e3)
         total += ms * 1e-3 * iters
     return statistics.median(per_call), min(per_call), len(per_call)
 
 
-def kernel_entry(kernel, arg_sets, nbytes, iters):
-    med, mn, blocks = time_kernel(kernel, arg_sets, iters)
+def kernel_entry(kernel, arg_sets, nbytes, iters, min_seconds=MIN_TIMED_SECONDS):
+    med, mn, blocks = time_kernel(kernel, arg_sets, iters, min_seconds)
     gbs = nbytes / (med * 1e-6) / 1e9
     return {
         "us": round(med, 2),
@@ -349,8 +392,10 @@ def cpu_baseline(params_kwargs, seed, sample_batch):
 # ------------------------------------------------------------------ workloads
 
 
-def bench_conv(args, device):
-    """One convolution shape: the fwd + backward step, its kernels, the yardsticks."""
+def bench_conv(args, device, workload=None, full=True):
+    """One convolution shape: the fwd + backward step, its kernels, the yardsticks.  `full=False`
+    (the compact entries of the default run's `configs` block) leaves out the graph replay, the
+    copy ceiling and the torch and CPU baselines, and times shorter blocks."""
     import torch
 
     from spio_amd.functional import fused_backward_kernel
@@ -361,7 +406,9 @@ def bench_conv(args, device):
         conv2d_gw8_wgrad_kernel_factory,
     )
 
-    desc, pkw, seed = WORKLOADS[args.workload]
+    workload = workload or args.workload
+    min_seconds = MIN_TIMED_SECONDS if full else MIN_TIMED_SECONDS / 4
+    desc, pkw, seed = WORKLOADS[workload]
     params = Conv2dGw8Params(**pkw)
     act_bytes = 2 * params.n * params.c * params.h * params.w
     out_bytes = 2 * params.n * params.c * params.p * params.q
@@ -398,7 +445,7 @@ def bench_conv(args, device):
         torch.cuda.synchronize()
         return time.perf_counter() - t
 
-    blocks = timed_blocks(block)
+    blocks = timed_blocks(block, min_seconds)
     ms_per_step = statistics.median(blocks) * 1e3 / args.steps
     ms_per_step_min = min(blocks) * 1e3 / args.steps
 
@@ -406,6 +453,8 @@ def bench_conv(args, device):
     # captures its training step gets; reported beside the eager figure, which stays `value`.
     graph_ms_per_step = None
     try:
+        if not full:
+            raise _Skip()
         graphs = []
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
@@ -429,6 +478,8 @@ def bench_conv(args, device):
 
         graph_ms_per_step = statistics.median(timed_blocks(gblock)) * 1e3 / args.steps
         del graphs
+    except _Skip:
+        pass
     except Exception as e:  # pylint: disable=broad-except
         print(f"bench.py: HIP graph replay skipped: {type(e).__name__}: {e}", file=sys.stderr)
 
@@ -447,13 +498,13 @@ def bench_conv(args, device):
     }
     nbytes["bgrad"] = nbytes["dgrad"] + nbytes["wgrad"] - out_bytes  # grad_output is read once
     kernels = {
-        "fprop": kernel_entry(k_fwd, [(s["y"], s["x"], w, None) for s in sets], nbytes["fprop"], iters),
-        "dgrad": kernel_entry(k_dgrad, [(s["dx"], s["dy"], w, None) for s in sets], nbytes["dgrad"], iters),
-        "wgrad": kernel_entry(k_wgrad, [(s["dw"], s["x"], s["dy"]) for s in sets], nbytes["wgrad"], iters),
+        "fprop": kernel_entry(k_fwd, [(s["y"], s["x"], w, None) for s in sets], nbytes["fprop"], iters, min_seconds),
+        "dgrad": kernel_entry(k_dgrad, [(s["dx"], s["dy"], w, None) for s in sets], nbytes["dgrad"], iters, min_seconds),
+        "wgrad": kernel_entry(k_wgrad, [(s["dw"], s["x"], s["dy"]) for s in sets], nbytes["wgrad"], iters, min_seconds),
     }
     if k_fused is not None:
         kernels["bgrad"] = kernel_entry(
-            k_fused, [(s["dx"], s["dw"], s["x"], s["dy"], w) for s in sets], nbytes["bgrad"], iters
+            k_fused, [(s["dx"], s["dw"], s["x"], s["dy"], w) for s in sets], nbytes["bgrad"], iters, min_seconds
         )
         kernels["bgrad"]["note"] = ("fused dgrad+wgrad as the backward op runs it for this shape; replaces "
                                     "the dgrad and wgrad launches in the timed step")
@@ -470,7 +521,9 @@ def bench_conv(args, device):
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
     dominant = max(in_step, key=lambda n: kernels[n]["us"])
     for name in kernels:
-        kernels[name]["traffic"] = measured_traffic(args.workload, name)
+        attach_profile_figures(kernels[name], workload, name)
+        # what an empty kernel costs in the same back-to-back loop, as a share of this kernel's time
+        kernels[name]["launch_floor_share"] = round(LAUNCH_FLOOR_US / kernels[name]["us"], 3)
     roofline = {
         "bound": "hbm",
         "kernel": kernels[dominant]["kernel"],
@@ -480,6 +533,24 @@ def bench_conv(args, device):
         "frac": kernels[dominant]["frac_of_hbm_peak"],
         "traffic": kernels[dominant]["traffic"],
     }
+    for key in ("traffic_stale", "mfma_util", "mfma_util_stale"):
+        if key in kernels[dominant]:
+            roofline[key] = kernels[dominant][key]
+    if not full:
+        del sets
+        torch.cuda.empty_cache()
+        compact = {}
+        for name, e in kernels.items():
+            compact[name] = {k: e[k] for k in ("us", "us_min", "GB/s", "frac_of_hbm_peak", "traffic", "traffic_stale",
+                                               "mfma_util", "launch_floor_share", "bytes") if k in e}
+            compact[name]["config"] = {k: v for k, v in e["config"].items() if v not in (0, None)}
+        return {
+            "workload": desc, "params": params.encode(), "step_kernels": in_step,
+            "step_us": round(ms_per_step * 1e3, 2), "step_GB/s": round(value, 1),
+            "step_frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4), "step_bytes": step_bytes,
+            "first_use_seconds": round(setup_s, 2), "buffer_sets": nsets, "kernels": compact,
+            "roofline": roofline,
+        }  # fmt: skip
 
     result = {
         "metric": METRIC,
@@ -536,7 +607,11 @@ def bench_conv(args, device):
     return result
 
 
-def bench_batch_sweep(args, device):
+class _Skip(Exception):
+    """Raised to leave out an optional measurement."""
+
+
+def bench_batch_sweep(args, device, full=True):
     """cfg4: the forward kernel (and the backward half) at C=64 56x56 3x3 for N = 1 .. 512: the
     reference's headline plot, effective bandwidth versus batch size
     (scripts/profile_blocks.bash:4-5, scripts/plot_kernel_bench.py:417-435)."""
@@ -557,25 +632,27 @@ def bench_batch_sweep(args, device):
         nsets = rotation_sets(2 * act)
         w, sets = make_buffers(params, 0, nsets, device)
         iters = 200 if n <= 64 else 60
+        min_seconds = MIN_TIMED_SECONDS if full else MIN_TIMED_SECONDS / 4
         k_fwd = conv2d_gw8_kernel_factory.get_kernel(params, device)
         fb = Conv2dStats(params, output_names="output").bytes
-        e = kernel_entry(k_fwd, [(s["y"], s["x"], w, None) for s in sets], fb, iters)
+        e = kernel_entry(k_fwd, [(s["y"], s["x"], w, None) for s in sets], fb, iters, min_seconds)
         point = {"N": n, "fprop_us": e["us"], "fprop_GB/s": e["GB/s"], "fprop_frac": e["frac_of_hbm_peak"],
-                 "fprop_bytes": fb, "launch_floor_dominated": e["us"] < 3 * LAUNCH_FLOOR_US}  # fmt: skip
+                 "fprop_bytes": fb, "launch_floor_dominated": e["us"] < 3 * LAUNCH_FLOOR_US,
+                 "fprop_launch_floor_share": round(LAUNCH_FLOOR_US / e["us"], 3)}  # fmt: skip
         k_fused = fused_backward_kernel(params, device)
         st_w = Conv2dStats(params, output_names="grad_weight")
         wb = st_w.bytes_read + st_w.grad_weight_bytes_written_fp32
         db = Conv2dStats(params, output_names="grad_input").bytes
         if k_fused is not None:
             bb = db + wb - act
-            b = kernel_entry(k_fused, [(s["dx"], s["dw"], s["x"], s["dy"], w) for s in sets], bb, iters)
+            b = kernel_entry(k_fused, [(s["dx"], s["dw"], s["x"], s["dy"], w) for s in sets], bb, iters, min_seconds)
             point.update({"backward": "fused", "backward_us": b["us"], "backward_GB/s": b["GB/s"],
                           "backward_frac": b["frac_of_hbm_peak"], "backward_bytes": bb})  # fmt: skip
         else:
             k_d = conv2d_gw8_kernel_factory.get_kernel(params, device, igrad=True)
             k_w = conv2d_gw8_wgrad_kernel_factory.get_kernel(params, device)
-            d = kernel_entry(k_d, [(s["dx"], s["dy"], w, None) for s in sets], db, iters)
-            ww = kernel_entry(k_w, [(s["dw"], s["x"], s["dy"]) for s in sets], wb, iters)
+            d = kernel_entry(k_d, [(s["dx"], s["dy"], w, None) for s in sets], db, iters, min_seconds)
+            ww = kernel_entry(k_w, [(s["dw"], s["x"], s["dy"]) for s in sets], wb, iters, min_seconds)
             us = d["us"] + ww["us"]
             point.update({"backward": "dgrad+wgrad", "backward_us": round(us, 2),
                           "backward_GB/s": round((db + wb) / us / 1e3, 1),
@@ -606,13 +683,12 @@ def bench_batch_sweep(args, device):
     }  # fmt: skip
 
 
-def bench_network(args, device):
+def bench_network(args, device, full=True):
     """cfg5: inference of the ConvNeXt-Tiny-shaped gw8 network at batch 128 (fp16 autocast, channels_last),
     with the time of its four distinct gw8 convolution shapes and of the channel LayerNorm."""
     import torch
 
-    sys.path.insert(0, os.path.join(ROOT, "tests"))
-    from convnext_gw8 import ConvNeXtGw8  # pylint: disable=import-error,import-outside-toplevel
+    from spio_amd.convnext_gw8 import ConvNeXtGw8
 
     from spio_amd.kernels import Conv2dGw8Params, Conv2dStats, conv2d_gw8_kernel_factory
     from spio_amd.layers import Conv2dGw8, LayerNorm2d
@@ -648,7 +724,7 @@ def bench_network(args, device):
             torch.cuda.synchronize()
             return time.perf_counter() - t
 
-        blocks = timed_blocks(block, min_seconds=1.0, max_blocks=20)
+        blocks = timed_blocks(block, min_seconds=1.0 if full else 0.3, max_blocks=20)
     ms_iter = statistics.median(blocks) * 1e3 / iters
 
     convs, total_bytes, total_us = [], 0, 0.0
@@ -659,9 +735,11 @@ def bench_network(args, device):
         nsets = rotation_sets(nb)
         k = conv2d_gw8_kernel_factory.get_kernel(params, device)
         asets = [conv2d_gw8_kernel_factory.make_test_args(params, device) for _ in range(nsets)]
-        e = kernel_entry(k, asets, nb, 100)
+        e = kernel_entry(k, asets, nb, 100, MIN_TIMED_SECONDS if full else MIN_TIMED_SECONDS / 4)
+        e["launch_floor_share"] = round(LAUNCH_FLOOR_US / e["us"], 3)
         convs.append({"shape": params.encode(), "count": depth[c], "us": e["us"], "GB/s": e["GB/s"],
-                      "frac_of_hbm_peak": e["frac_of_hbm_peak"], "bytes": nb})  # fmt: skip
+                      "frac_of_hbm_peak": e["frac_of_hbm_peak"], "bytes": nb,
+                      "launch_floor_share": e["launch_floor_share"]})  # fmt: skip
         total_bytes += depth[c] * nb
         total_us += depth[c] * e["us"]
         del asets
@@ -673,7 +751,7 @@ def bench_network(args, device):
         nb = 4 * batch * c * hw * hw + 8 * c
         nsets = rotation_sets(nb)
         asets = [layernorm_2d_kernel_factory.make_test_args(p, device) for _ in range(nsets)]
-        e = kernel_entry(k, asets, nb, 100)
+        e = kernel_entry(k, asets, nb, 100, MIN_TIMED_SECONDS if full else MIN_TIMED_SECONDS / 4)
         entry = {"shape": p.encode(), "us": e["us"], "GB/s": e["GB/s"],
                  "frac_of_hbm_peak": e["frac_of_hbm_peak"], "bytes": nb}  # fmt: skip
         del asets
@@ -684,7 +762,7 @@ def bench_network(args, device):
         nbb = 6 * batch * c * hw * hw + 4 * c
         nsets = rotation_sets(nbb)
         asets = [layernorm_2d_bwd_kernel_factory.make_test_args(pb, device) for _ in range(nsets)]
-        eb = kernel_entry(kb, asets, nbb, 100)
+        eb = kernel_entry(kb, asets, nbb, 100, MIN_TIMED_SECONDS if full else MIN_TIMED_SECONDS / 4)
         entry["backward"] = {"us": eb["us"], "GB/s": eb["GB/s"], "frac_of_hbm_peak": eb["frac_of_hbm_peak"],
                              "bytes": nbb}  # fmt: skip
         norms.append(entry)
@@ -713,7 +791,7 @@ def bench_network(args, device):
                      "achieved": slowest["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": slowest["frac_of_hbm_peak"], "traffic": None},
     }  # fmt: skip
-    if not args.no_cpu_baseline:
+    if full and not args.no_cpu_baseline:
         sample = 2
         torch.manual_seed(3)
         cpu_model = ConvNeXtGw8().float().eval()
@@ -735,6 +813,92 @@ def bench_network(args, device):
             "logical_cpus": os.cpu_count(), "physical_cores": physical_cores(),
         }  # fmt: skip
     return result
+
+
+def precompile_recorded_kernels():
+    """Compiles, in the compiler's thread pool, the recorded configuration of every kernel the
+    `configs` block will ask for; the code objects land in the on-disk cache, so the requests
+    that follow load them instead of compiling one after the other."""
+    from spio_amd.compiler.compiler_pool import compile_kernels
+    from spio_amd.hip import get_device_attributes
+    from spio_amd.kernels import (
+        Conv2dGw8Params,
+        conv2d_gw8_bgrad_kernel_factory,
+        conv2d_gw8_kernel_factory,
+        conv2d_gw8_wgrad_kernel_factory,
+    )
+    from spio_amd.kernels.layernorm_2d_kernel import (
+        LayerNorm2dParams,
+        layernorm_2d_bwd_kernel_factory,
+        layernorm_2d_kernel_factory,
+    )
+    from spio_amd.kernels.tuner import tuner
+
+    attr = get_device_attributes(0)
+    conv_families = ((conv2d_gw8_kernel_factory, {}), (conv2d_gw8_kernel_factory, {"igrad": True}),
+                     (conv2d_gw8_wgrad_kernel_factory, {}), (conv2d_gw8_bgrad_kernel_factory, {}))  # fmt: skip
+    requests = []
+    shapes = [Conv2dGw8Params(**WORKLOADS[w][1]) for w in ("cfg1", "cfg2", "cfg3")]
+    shapes += [Conv2dGw8Params(n=n, c=64, h=56, w=56, padding=1, r=3, s=3) for n in SWEEP_BATCHES]
+    for params in shapes:
+        requests += [(f, params, kw) for f, kw in conv_families]
+    for c, hw in NETWORK_WIDTHS:
+        requests.append((conv2d_gw8_kernel_factory, Conv2dGw8Params(n=128, c=c, h=hw, w=hw, padding=1, has_bias=True), {}))
+        requests.append((layernorm_2d_kernel_factory, LayerNorm2dParams(n=128, c=c, h=hw, w=hw), {}))
+        requests.append((layernorm_2d_bwd_kernel_factory, LayerNorm2dParams(n=128, c=c, h=hw, w=hw, has_bias=False), {}))
+    kernels = []
+    for factory, params, kw in requests:
+        try:
+            record = tuner.lookup(attr, factory.get_full_kernel_name(params, **kw))
+            if record is None:
+                continue
+            config = factory.config_cls(**record["config"])
+            if config in list(factory.configs(params, attr, **kw)):
+                kernels.append(factory.make_kernel(params, config, attr, **kw))
+        except Exception:  # pylint: disable=broad-except
+            continue
+    try:
+        compile_kernels(kernels)
+    except ValueError as e:
+        print(f"bench.py: precompilation failed, kernels compile on first use: {e}", file=sys.stderr)
+    return len(kernels)
+
+
+def configs_block(args, device):
+    """Compact measurements of every BASELINE configuration next to the headline workload."""
+    import torch
+
+    t0 = time.perf_counter()
+    out = {"precompiled_kernels": precompile_recorded_kernels()}
+    out["precompile_seconds"] = round(time.perf_counter() - t0, 1)
+    for name in ("cfg1", "cfg2", "cfg3"):
+        t = time.perf_counter()
+        try:
+            out[name] = bench_conv(args, device, workload=name, full=False)
+            out[name]["seconds"] = round(time.perf_counter() - t, 1)
+        except Exception as e:  # pylint: disable=broad-except
+            out[name] = {"error": f"{type(e).__name__}: {e}"[:300]}
+        torch.cuda.empty_cache()
+    t = time.perf_counter()
+    try:
+        sweep = bench_batch_sweep(args, device, full=False)
+        out["cfg4"] = {"workload": sweep["config"]["workload"], "sweep": sweep["sweep"], "note": sweep["note"],
+                       "seconds": round(time.perf_counter() - t, 1)}  # fmt: skip
+    except Exception as e:  # pylint: disable=broad-except
+        out["cfg4"] = {"error": f"{type(e).__name__}: {e}"[:300]}
+    torch.cuda.empty_cache()
+    t = time.perf_counter()
+    try:
+        net = bench_network(args, device, full=False)
+        out["cfg5"] = {k: net[k] for k in ("network_ms_per_iter", "images_per_second", "gw8_conv_ms_per_iter",
+                                           "convs", "layernorm_2d", "frac_of_hbm_peak")}  # fmt: skip
+        out["cfg5"]["workload"] = net["config"]["workload"]
+        out["cfg5"]["seconds"] = round(time.perf_counter() - t, 1)
+    except Exception as e:  # pylint: disable=broad-except
+        out["cfg5"] = {"error": f"{type(e).__name__}: {e}"[:300]}
+    torch.cuda.empty_cache()
+    out["seconds"] = round(time.perf_counter() - t0, 1)
+    return out
 
 
 def main():
@@ -760,6 +924,8 @@ def main():
         result = bench_network(args, device)
     else:
         result = bench_conv(args, device)
+        if args.workload == "target" and not args.no_configs:
+            result["configs"] = configs_block(args, device)
     print(json.dumps(result))
 
 

@@ -1,6 +1,6 @@
 """ConvNeXt-Tiny-shaped network whose 7x7 depthwise convolutions are replaced by 3x3 convolutions
-with group width 8 (the fifth benchmark configuration).  This is test material: the reference
-ships no such model.  Stages of widths 96/192/384/768 at 56/28/14/7 spatial for 224x224 inputs,
+with group width 8 (the fifth benchmark configuration), for the benchmark and the tests.  The
+reference ships no such model (its nearest relative is the block in scripts/profile_block.py:75-114).  Stages of widths 96/192/384/768 at 56/28/14/7 spatial for 224x224 inputs,
 depths 3/3/9/3, LayerNorm + 4x MLP + GELU, 1000-class head.  Layer scale is initialised to 1 (not
 the usual 1e-6) so that the convolutions reach the logits and a wrong convolution shows."""
 

@@ -54,6 +54,15 @@ using namespace spio;
 #ifndef SPIO_PF
 #define SPIO_PF 2
 #endif
+#ifndef SPIO_PF0
+#define SPIO_PF0 SPIO_PF
+#endif
+#ifndef SPIO_PF_RATE
+#define SPIO_PF_RATE 1
+#endif
+#ifndef SPIO_BP2
+#define SPIO_BP2 0
+#endif
 #ifndef SPIO_TS
 #define SPIO_TS 1
 #endif
@@ -77,9 +86,26 @@ constexpr int EPX = kIgrad ? kS - 1 - kPadX : kPadX;
 
 constexpr int GB = SPIO_GB;  // groups (waves along channels) per workgroup
 constexpr int BP = SPIO_BP;  // output rows per workgroup
+// Two tile heights (SPIO_BP2 > 0): the row blocks of an image alternate between BP and BP2 rows;
+// the first half of the grid takes the BP-row tiles and the second half the BP2-row tiles.  A
+// grid of two workgroups per compute unit is dispatched as two cohorts (ids below half the grid
+// land one per CU first, the rest join them a moment later); memory serves requests in arrival
+// order, so the first cohort's prefetch burst is served before the second cohort's first row,
+// the second cohort trails by that burst for the whole kernel and then finishes alone at one
+// workgroup per CU (measured at N=128, C=64, 56x56 with equal tiles: 13.3 us against 18.0 us).
+// Taller tiles for the leading cohort and shorter ones for the trailing one let both end together.
+constexpr int BP2 = SPIO_BP2;
 constexpr int NB = SPIO_NB;  // images per workgroup
 constexpr int TS = SPIO_TS;  // waves sharing the tiles of one group
-constexpr int PF = SPIO_PF;  // prefetch distance in rows
+constexpr int PF = SPIO_PF;  // prefetch distance in rows (register buffers for rows in flight)
+// The distance is reached by a ramp: PF0 rows are requested before the first step and PF_RATE
+// rows per step from then on until the requests run PF rows ahead.  All workgroups of a launch
+// start within a fraction of a microsecond of each other and memory serves requests roughly in
+// the order they arrive; a workgroup that asks for all PF rows at once gets them before a
+// workgroup that started a moment later gets its first row, and the late ones then finish long
+// after the others.  With a short first burst every workgroup has its first rows early.
+constexpr int PF0 = SPIO_PF0 < SPIO_PF ? SPIO_PF0 : SPIO_PF;
+constexpr int PF_RATE = SPIO_PF_RATE;
 constexpr int WAVES = GB * TS;
 constexpr int THREADS = 64 * WAVES;
 
@@ -102,10 +128,11 @@ constexpr int LPT = (IN_CELLS + THREADS - 1) / THREADS;  // source cells per thr
 constexpr int OUT_CELLS = NB * DW * GB;
 constexpr int SPT = (OUT_CELLS + THREADS - 1) / THREADS;  // stores per thread per row
 constexpr int GBLKS = (kGroups + GB - 1) / GB;
-constexpr int PBLKS = (DH + BP - 1) / BP;
+constexpr int PAIRS = (DH + BP + BP2 - 1) / (BP + BP2);  // (BP, BP2) pairs of row blocks per image
+constexpr int PBLKS = BP2 > 0 ? PAIRS : (DH + BP - 1) / BP;  // row blocks of one height per image
 constexpr int NBLKS = (kN + NB - 1) / NB;
-constexpr int NUM_BLOCKS = GBLKS * PBLKS * NBLKS;
-constexpr int STEPS = BP + kR - 1;
+constexpr int HALF_BLOCKS = GBLKS * PBLKS * NBLKS;  // workgroups per tile height
+constexpr int NUM_BLOCKS = (BP2 > 0 ? 2 : 1) * HALF_BLOCKS;
 
 // The step loop is unrolled completely: every rotation index and every "is there a row to load
 // / to store" is then a compile-time fact, and no memory instruction sits in a loop whose entry
@@ -113,8 +140,8 @@ constexpr int STEPS = BP + kR - 1;
 #ifndef SPIO_MAX_UNROLL
 #define SPIO_MAX_UNROLL 64
 #endif
-static_assert(STEPS <= SPIO_MAX_UNROLL, "block_p + R - 1 exceeds the unrolled step limit");
-static_assert(PF >= 2 && WAVES <= 16, "bad configuration");
+static_assert((BP > BP2 ? BP : BP2) + kR - 1 <= SPIO_MAX_UNROLL, "block_p + R - 1 exceeds the unrolled step limit");
+static_assert(PF >= 2 && PF0 >= 2 && PF_RATE >= 1 && WAVES <= 16, "bad configuration");
 constexpr int STREAM_UNITS = NR * RING_ROW_UNITS + 2 * OUT_ROW_BYTES / 16;
 constexpr int FILTER_UNITS = kIgrad ? GB * 8 * kR * kS : 0;  // staged filters (data gradient only)
 constexpr int LDS_UNITS = STREAM_UNITS > FILTER_UNITS ? STREAM_UNITS : FILTER_UNITS;
@@ -128,6 +155,9 @@ static_assert(NB * SRC_IMAGE_BYTES < (1ll << 31) && NB * DST_IMAGE_BYTES < (1ll 
 constexpr unsigned OOB = 0x80000000u;  // offset of a lane without data: beyond every descriptor
 
 constexpr int pmod(int a, int m) { return ((a % m) + m) % m; }
+constexpr int cmin(int a, int b) { return a < b ? a : b; }
+// Source rows requested once step t of `steps` has issued its loads (t = -1: before the first step).
+constexpr int rows_requested(int t, int steps) { return cmin(cmin(steps, t + 1 + PF), PF0 + PF_RATE * (t + 1)); }
 
 // Source rows shared with the neighbouring row blocks (the first and last R-1
 // steps) can be served from L2 when the neighbour runs on the same XCD;
@@ -136,26 +166,38 @@ constexpr int pmod(int a, int m) { return ((a % m) + m) % m; }
 #ifndef SPIO_HALO_CACHED
 #define SPIO_HALO_CACHED 0
 #endif
-constexpr int AUX_NT = SPIO_NT ? 2 : 0;  // cache-policy operand of the buffer instructions
+// Cache-policy operands of the buffer instructions (gfx950: 1 = sc0, 2 = nt, 16 = sc1), one for
+// the interior source rows, one for the rows shared with neighbouring row blocks, one for the
+// stores.  SPIO_NT = 1 streams with the non-temporal hint unless a policy is given explicitly.
+#ifndef SPIO_LD_POLICY
+#define SPIO_LD_POLICY (SPIO_NT ? 2 : 0)
+#endif
+#ifndef SPIO_ST_POLICY
+#define SPIO_ST_POLICY (SPIO_NT ? 2 : 0)
+#endif
+#ifndef SPIO_HALO_POLICY
+#define SPIO_HALO_POLICY (SPIO_HALO_CACHED ? 0 : SPIO_LD_POLICY)
+#endif
+constexpr int AUX_LD = SPIO_LD_POLICY;
+constexpr int AUX_HALO = SPIO_HALO_POLICY;
+constexpr int AUX_ST = SPIO_ST_POLICY;
 
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
 SPIO_DEVICE rsrc_t make_rsrc(const void* base, int bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
 }
 
-}  // namespace
+// pointers typed in the LDS address space: 32-bit address arithmetic, constant parts of an
+// index end up in the instruction's offset field
+typedef __attribute__((address_space(3))) spio_uint4* lds_u4p;
+typedef __attribute__((address_space(3))) unsigned char* lds_bytep;
 
-extern "C" __global__ void SPIO_LAUNCH_BOUNDS(THREADS)
-SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ src,
-                 const spio_half* __restrict__ weights, const float* __restrict__ bias) {
-    // One LDS block: the source-row ring, then the two output-stage rows.  The data-gradient
-    // mode first uses the same block to stage the filters of the workgroup's groups.
-    __shared__ spio_uint4 lds[LDS_UNITS];
-    // pointers typed in the LDS address space: 32-bit address arithmetic, constant parts of an
-    // index end up in the instruction's offset field
-    typedef __attribute__((address_space(3))) spio_uint4* lds_u4p;
-    typedef __attribute__((address_space(3))) unsigned char* lds_bytep;
-    const lds_u4p ring = (lds_u4p)lds;
+// One tile: ROWS output rows starting at row p0 of the NB images from n0 on, channel block cb.
+template <int ROWS>
+SPIO_DEVICE void conv_rows(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ src,
+                           const spio_half* __restrict__ weights, const float* __restrict__ bias,
+                           const lds_u4p ring, const int p0, const int n0, const int cb) {
+    constexpr int STEPS = ROWS + kR - 1;
     const lds_bytep ostage = (lds_bytep)(ring + NR * RING_ROW_UNITS);
 
     const int tid = thread_id();
@@ -164,35 +206,6 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wg = wave % GB;  // group within the workgroup
     const int ws = wave / GB;  // tile split index
-
-    // Workgroup -> (image block, channel block, row block), row block fastest.
-    // Consecutive workgroup ids are dealt round-robin to the 8 XCDs.  Remap so that runs of
-    // SPIO_XCD_CHUNK consecutive tiles land on one XCD (neighbouring row blocks share halo rows
-    // through that XCD's L2) while the tiles in flight on the whole device at any moment still
-    // form one compact, advancing range of addresses (HBM streams best through such a front;
-    // eight distant fronts, one per XCD, cost several per cent).  0 = one contiguous range of
-    // tiles per XCD.
-    int b = block_id();
-    {
-        constexpr int CH = SPIO_XCD_CHUNK;
-        if (CH == 0) {
-            if (NUM_BLOCKS % 8 == 0) b = (b & 7) * (NUM_BLOCKS / 8) + (b >> 3);
-        } else if (CH > 1 && NUM_BLOCKS % (8 * CH) == 0) {
-            const int x = b & 7;   // XCD
-            const int k = b >> 3;  // position in that XCD's sequence
-            b = (k / CH) * (8 * CH) + x * CH + k % CH;
-        }
-    }
-    // Tile order: row blocks fastest, so that neighbours in a run share halo rows.  Where a
-    // workgroup covers only part of a pixel's 128-byte lines (GB * 16 bytes per pixel), the channel
-    // blocks that share those lines go fastest instead: dealt to different XCDs, every one of
-    // them would fetch the whole lines from memory (measured: twice the algorithmic reads).
-    constexpr bool kSplitLines = GBLKS > 1 && (GB * 16) % 128 != 0;
-    const int pb = kSplitLines ? (b / GBLKS) % PBLKS : b % PBLKS;
-    const int cb = kSplitLines ? b % GBLKS : (b / PBLKS) % GBLKS;
-    const int nb = b / (PBLKS * GBLKS);
-    const int p0 = pb * BP;
-    const int n0 = nb * NB;
     const int gglob = cb * GB + wg;
     const bool wave_active = gglob < kGroups;  // idle waves compute on zeros and store nothing
 
@@ -240,13 +253,12 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
         // (readfirstlane: the row offset must stay in a scalar register whatever the optimiser
         //  makes of the clamp)
         const int soff = __builtin_amdgcn_readfirstlane(imin(imax(h, 0), SH - 1) * SRC_ROW_BYTES);
-        const bool halo = t < kR - 1 || t >= BP;
+        const bool halo = t < kR - 1 || t >= ROWS;
 #pragma unroll
         for (int l = 0; l < LPT; ++l) {
             Pack16 v;
-            v.i = (SPIO_HALO_CACHED && halo)
-                      ? __builtin_amdgcn_raw_buffer_load_b128(rs, (int)in_voff[l], soff, 0)
-                      : __builtin_amdgcn_raw_buffer_load_b128(rs, (int)in_voff[l], soff, AUX_NT);
+            v.i = halo ? __builtin_amdgcn_raw_buffer_load_b128(rs, (int)in_voff[l], soff, AUX_HALO)
+                       : __builtin_amdgcn_raw_buffer_load_b128(rs, (int)in_voff[l], soff, AUX_LD);
             regs[l] = v.u;
         }
     };
@@ -296,7 +308,7 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
     // ---- rows 0..PF-1 into registers: their latency covers the rest of the set-up ----
     spio_uint4 pre[PF][LPT];
 #pragma unroll
-    for (int t = 0; t < PF; ++t) load_row(pre[t], imin(t, STEPS - 1));
+    for (int t = 0; t < PF0; ++t) load_row(pre[t], imin(t, STEPS - 1));
     __builtin_amdgcn_sched_barrier(0);  // ... and the row loads ahead of everything that waits
 
     // ---- loop-invariant addressing of the cooperative row store ----
@@ -433,7 +445,7 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
         for (int s = 0; s < SPT; ++s) {
             Pack16 v;
             v.u = *(lds_u4p)(ostage + obuf * OUT_ROW_BYTES + out_lds[s]);
-            __builtin_amdgcn_raw_buffer_store_b128(v.i, rs, (int)(out_voff[s] + row_off), 0, AUX_NT);
+            __builtin_amdgcn_raw_buffer_store_b128(v.i, rs, (int)(out_voff[s] + row_off), 0, AUX_ST);
         }
     };
 
@@ -464,10 +476,11 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
     for (int t = 0; t < STEPS; ++t) {
         const int ph = t % NS;    // all of these are compile-time constants after unrolling
         const int obuf = t & 1;   // output stage buffer of this step
-        const int pbuf = t % PF;  // register buffer that held row t
 
-        // 1. prefetch source row t+PF (its register buffer is free: row t is in LDS)
-        if (t + PF < STEPS) load_row(pre[pbuf], t + PF);
+        // 1. prefetch the next source rows, at most up to row t+PF (whose register buffer is
+        //    free: row t is in LDS)
+#pragma unroll
+        for (int r = rows_requested(t - 1, STEPS); r < rows_requested(t, STEPS); ++r) load_row(pre[r % PF], r);
 
         // 2. fragment reads of this step's row; the previous step's output row is stored while
         //    they are in flight
@@ -528,4 +541,57 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
         block_sync();
     }
     store_output_row(STEPS - 1, (STEPS - 1) & 1);  // the last row
+}
+
+}  // namespace
+
+extern "C" __global__ void SPIO_LAUNCH_BOUNDS(THREADS)
+SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ src,
+                 const spio_half* __restrict__ weights, const float* __restrict__ bias) {
+    // One LDS block: the source-row ring, then the two output-stage rows.  The data-gradient
+    // mode first uses the same block to stage the filters of the workgroup's groups.
+    __shared__ spio_uint4 lds[LDS_UNITS];
+    const lds_u4p ring = (lds_u4p)lds;
+
+    // Workgroup -> (image block, channel block, row block), row block fastest.
+    // Consecutive workgroup ids are dealt round-robin to the 8 XCDs.  Remap so that runs of
+    // SPIO_XCD_CHUNK consecutive tiles land on one XCD (neighbouring row blocks share halo rows
+    // through that XCD's L2) while the tiles in flight on the whole device at any moment still
+    // form one compact, advancing range of addresses (HBM streams best through such a front;
+    // eight distant fronts, one per XCD, cost several per cent).  0 = one contiguous range of
+    // tiles per XCD.
+    // With two tile heights the two halves of the grid are two such sequences of tiles, one per
+    // height, and a tile and the one below it (the other height) have the same index in both:
+    // their workgroups run on the same XCD and share their halo rows.
+    const int raw = block_id();
+    const bool second = BP2 > 0 && raw >= HALF_BLOCKS;
+    int b = second ? raw - HALF_BLOCKS : raw;
+    {
+        constexpr int CH = SPIO_XCD_CHUNK;
+        if (CH == 0) {
+            if (HALF_BLOCKS % 8 == 0) b = (b & 7) * (HALF_BLOCKS / 8) + (b >> 3);
+        } else if (CH > 1 && HALF_BLOCKS % (8 * CH) == 0) {
+            const int x = b & 7;   // XCD
+            const int k = b >> 3;  // position in that XCD's sequence
+            b = (k / CH) * (8 * CH) + x * CH + k % CH;
+        }
+    }
+    // Tile order: row blocks fastest, so that neighbours in a run share halo rows.  Where a
+    // workgroup covers only part of a pixel's 128-byte lines (GB * 16 bytes per pixel), the channel
+    // blocks that share those lines go fastest instead: dealt to different XCDs, every one of
+    // them would fetch the whole lines from memory (measured: twice the algorithmic reads).
+    constexpr bool kSplitLines = GBLKS > 1 && (GB * 16) % 128 != 0;
+    const int pb = kSplitLines ? (b / GBLKS) % PBLKS : b % PBLKS;
+    const int cb = kSplitLines ? b % GBLKS : (b / PBLKS) % GBLKS;
+    const int nb = b / (PBLKS * GBLKS);
+    const int n0 = nb * NB;
+    if (BP2 > 0) {
+        const int p0 = pb * (BP + BP2);
+        if (second)
+            conv_rows<(BP2 > 0 ? BP2 : 1)>(dst, src, weights, bias, ring, p0 + BP, n0, cb);
+        else
+            conv_rows<BP>(dst, src, weights, bias, ring, p0, n0, cb);
+    } else {
+        conv_rows<BP>(dst, src, weights, bias, ring, pb * BP, n0, cb);
+    }
 }

@@ -31,12 +31,11 @@ MAX_LDS_BYTES = 128 * 1024
 MAX_UNROLLED_STEPS = 64  # SPIO_MAX_UNROLL of the kernel: up to here the step loop is fully unrolled
 MAX_LOADS_PER_THREAD = 8
 MAX_ACCUMULATORS = 16
-MAX_CONFIGS = 36
 DEVICE_LDS_BYTES = 160 * 1024
 MAX_IMAGE_CONFIGS = 10  # whole-image configurations that enter the sweep
 MOVER_WAVES = 4  # data-mover waves of the whole-image kernel where it has any: one per SIMD
-PREFETCH_CHOICES = (2, 4, 8, 12, 16)
-MAX_GEOMETRIES = 24  # tile geometries that enter the sweep; the best few also try the other cache/XCD policies
+PREFETCH_CHOICES = (2, 4, 8, 10, 12, 16)
+MAX_GEOMETRIES = 30  # tile geometries that enter the sweep; the best few also try the other cache/XCD policies
 
 
 @dataclass(frozen=True)
@@ -66,6 +65,14 @@ class Conv2dGw8Config:
         movers: whole-image kernel only: extra waves that move the image blocks between global
             memory and LDS for the whole workgroup while the other waves only multiply (0: every
             wave does both).
+        block_p2: row-streaming kernel only: a second tile height.  The row blocks of an image
+            then alternate between block_p and block_p2 rows, the first half of the grid takes
+            the block_p tiles and the second half the block_p2 tiles.  For grids of two
+            workgroups per compute unit, which the device starts as two cohorts of which the
+            second trails the first by the first's prefetch burst (0: one height).
+        prefetch_start, prefetch_rate: row-streaming kernel only: rows requested before the
+            first step and per step until the requests run `prefetch` rows ahead
+            (prefetch_start = 0: all `prefetch` rows at once).
     """
 
     groups: int = 8
@@ -79,6 +86,9 @@ class Conv2dGw8Config:
     xcd_chunk: int = 4
     block_n_iters: int = 1
     movers: int = 0
+    block_p2: int = 0
+    prefetch_start: int = 0
+    prefetch_rate: int = 1
 
 
 def direction_geometry(params: Conv2dGw8Params, igrad: bool) -> Dict[str, int]:
@@ -95,6 +105,7 @@ def mfma_geometry(params: Conv2dGw8Params, config: Conv2dGw8Config, igrad: bool)
     d = direction_geometry(params, igrad)
     r, s = params.r, params.s
     gb, bp, nb, ts, pf = config.groups, config.block_p, config.block_n, config.split, config.prefetch
+    bp2 = config.block_p2
     ns = 2 * ((r + 1) // 2)
     kb = (s + 3) // 4
     wpi = d["DW"] + s - 1
@@ -111,10 +122,12 @@ def mfma_geometry(params: Conv2dGw8Params, config: Conv2dGw8Config, igrad: bool)
         NS=ns, NACC=ns // 2, KB=kb, WPI=wpi, F=f, WT=wt, TPW=divup(wt, ts), GS=gs,
         THREADS=threads, LDS_BYTES=lds, LPT=divup(f * gb, threads),
         SPT=divup(nb * d["DW"] * gb, threads),
-        GBLKS=divup(params.groups, gb), PBLKS=divup(d["DH"], bp), NBLKS=divup(params.n, nb),
-        STEPS=bp + r - 1, UNROLL=ns // gcd(ns, pf) * pf,
+        GBLKS=divup(params.groups, gb), NBLKS=divup(params.n, nb),
+        # two tile heights: PBLKS (block_p, block_p2) pairs per image, one workgroup per tile
+        PBLKS=divup(d["DH"], bp + bp2) if bp2 else divup(d["DH"], bp),
+        STEPS=max(bp, bp2) + r - 1, UNROLL=ns // gcd(ns, pf) * pf,
     )  # fmt: skip
-    d["NUM_BLOCKS"] = d["GBLKS"] * d["PBLKS"] * d["NBLKS"]
+    d["NUM_BLOCKS"] = (2 if bp2 else 1) * d["GBLKS"] * d["PBLKS"] * d["NBLKS"]
     return d
 
 
@@ -236,6 +249,11 @@ def _mfma_config_is_legal(params, config, igrad) -> bool:
         and config.split <= g["WT"]
         and config.block_n <= max(params.n, 1)
         and config.block_p <= g["DH"]
+        and config.block_p2 >= 0
+        and (config.block_p2 == 0 or config.block_p + config.block_p2 <= g["DH"])
+        and 0 <= config.prefetch_start <= config.prefetch
+        and config.prefetch_start != 1
+        and config.prefetch_rate >= 1
         and g["LDS_BYTES"] <= MAX_LDS_BYTES
         and g["LPT"] <= MAX_LOADS_PER_THREAD
         and g["TPW"] * g["NACC"] <= MAX_ACCUMULATORS
@@ -274,12 +292,43 @@ def _mfma_score(params, config, igrad, num_cus: int) -> float:
     in_flight = resident * min(config.prefetch, g["STEPS"]) * row_bytes
     starve = 1.0 + 0.6 * max(0.0, (64 * 1024 - in_flight) / (64 * 1024))
     few_waves = 1.15 if resident * g["THREADS"] < 512 else 1.0
+    # one workgroup on a CU has nothing to run while it waits at its barrier (measured at N=128,
+    # C=64, 56x56: 28-row tiles, one per CU, 20.6 us; 14-row tiles, two per CU, 18.8 us)
+    alone = 1.04 if resident == 1 else 1.0
     big_block = 1.08 if g["THREADS"] > 512 else 1.0
     # a workgroup that covers only part of a 128-byte line of a pixel shares it with another one
     split_line = 1.0 if (config.groups * 16) % 128 == 0 or config.groups == params.groups else 1.12
     # every row block runs block_p steps, also the last, partly empty one
-    ragged = g["PBLKS"] * config.block_p / g["DH"]
-    return traffic * quant * ragged * starve * few_waves * big_block * split_line / (tile_eff ** 0.3 * group_eff)
+    ragged = g["PBLKS"] * (config.block_p + config.block_p2) / g["DH"]
+    return traffic * quant * ragged * starve * few_waves * alone * big_block * split_line / (tile_eff ** 0.3 * group_eff)
+
+
+def _two_height_configs(params, configs, igrad, num_cus) -> List[Conv2dGw8Config]:
+    """Variants of the leading geometries with two tile heights, for grids that put exactly two
+    workgroups on every compute unit in one round: the device starts such a grid as two cohorts
+    and the second trails the first by the first's prefetch burst, so the first half of the
+    grid gets taller tiles and the second half shorter ones (measured at N=128, C=64, 56x56:
+    14+14 rows 18.8 us, 19+9 rows 18.3 us).  The sweep decides; they rank behind the uniform
+    tiles so that a capped sweep is not spent on them."""
+    out = []
+    seen = set()
+    for cfg in configs:
+        shape = (cfg.groups, cfg.block_p, cfg.block_n, cfg.split)
+        if len(seen) == 2 or shape in seen:
+            continue
+        g = mfma_geometry(params, cfg, igrad)
+        if cfg.variant != "mfma" or cfg.block_p2 or g["NUM_BLOCKS"] != 2 * num_cus:
+            continue
+        if g["PBLKS"] % 2 or g["DH"] % (2 * cfg.block_p) or cfg.block_p < 4:
+            continue
+        seen.add(shape)
+        for frac in (0.29, 0.36, 0.43):
+            delta = max(1, round(cfg.block_p * frac))
+            for pf in sorted({cfg.prefetch, 10, 12}):
+                cand = replace(cfg, block_p=cfg.block_p + delta, block_p2=cfg.block_p - delta, prefetch=pf)
+                if cand not in out and _mfma_config_is_legal(params, cand, igrad):
+                    out.append(cand)
+    return out
 
 
 def _get_configs(params: Conv2dGw8Params, device_attr=None, igrad: bool = False) -> List[Conv2dGw8Config]:
@@ -305,10 +354,18 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None, igrad: bool = False)
     configs = [cfg for _, cfg in found[:MAX_GEOMETRIES]]
     # the memory-system policies, which the score cannot rank: halo rows with or without the
     # non-temporal hint, and how tiles are dealt to the XCDs
-    for cfg in list(configs[:4]):
-        for hc, ch in ((0, 4), (1, 0), (0, 0)):
-            configs.append(replace(cfg, halo_cached=hc, xcd_chunk=ch))
-    configs = configs[:MAX_CONFIGS]
+    leading = []  # the first four tile geometries, whatever their prefetch depth
+    for cfg in configs:
+        shape = (cfg.groups, cfg.block_p, cfg.block_n, cfg.split)
+        if shape not in leading:
+            if len(leading) == 4:
+                break
+            leading.append(shape)
+    for cfg in list(configs):
+        if (cfg.groups, cfg.block_p, cfg.block_n, cfg.split) in leading:
+            for hc, ch in ((0, 4), (1, 0), (0, 0)):
+                configs.append(replace(cfg, halo_cached=hc, xcd_chunk=ch))
+    configs += _two_height_configs(params, configs, igrad, num_cus)
     # small images: the whole-image kernel; its two best candidates go first, so that the capped
     # sweep an operator runs on an unrecorded shape sees both kernels
     image = _image_configs(params, igrad, num_cus)
@@ -362,6 +419,12 @@ def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8Config, _device_a
         SPIO_NT=config.nontemporal, SPIO_HALO_CACHED=config.halo_cached,
         SPIO_XCD_CHUNK=config.xcd_chunk,
     )  # fmt: skip
+    if config.block_p2:
+        defines["SPIO_BP2"] = config.block_p2
+    if config.prefetch_start:
+        defines["SPIO_PF0"] = config.prefetch_start
+    if config.prefetch_rate != 1:
+        defines["SPIO_PF_RATE"] = config.prefetch_rate
     return KernelSpec(
         defines, LaunchParams(grid=g["NUM_BLOCKS"], block=g["THREADS"]), MFMA_SOURCE, notes=g
     )

@@ -35,10 +35,14 @@ class LayerNorm2dParams:
     has_bias: bool = True
 
     def encode(self) -> str:
+        """The name is part of the kernel's symbol, so it holds identifier characters only: eps is
+        its shortest round-trip decimal form with '.' written 'p', '-' written 'm' and '+' dropped
+        (1e-06 -> 1em06, 0.001 -> 0p001, 1.5e-05 -> 1p5em05)."""
         flags = ("w" if self.has_weight else "nw") + ("b" if self.has_bias else "nb")
-        return f"{self.n}n_{self.c}c_{self.h}h_{self.w}w_{self.eps:g}eps_{flags}".replace("-", "m")
+        eps = repr(float(self.eps)).replace(".", "p").replace("-", "m").replace("+", "")
+        return f"{self.n}n_{self.c}c_{self.h}h_{self.w}w_{eps}eps_{flags}"
 
-    _PATTERN = re.compile(r"(\d+)n_(\d+)c_(\d+)h_(\d+)w_([0-9.em+]+)eps_(w|nw)(b|nb)$")
+    _PATTERN = re.compile(r"(\d+)n_(\d+)c_(\d+)h_(\d+)w_([0-9epm]+)eps_(w|nw)(b|nb)$")
 
     @classmethod
     def decode(cls, string: str) -> "LayerNorm2dParams":
@@ -46,7 +50,7 @@ class LayerNorm2dParams:
         if m is None:
             raise ValueError("Invalid string representation.")
         n, c, h, w = (int(v) for v in m.groups()[:4])
-        return cls(n=n, c=c, h=h, w=w, eps=float(m.group(5).replace("m", "-")),
+        return cls(n=n, c=c, h=h, w=w, eps=float(m.group(5).replace("p", ".").replace("m", "-")),
                    has_weight=m.group(6) == "w", has_bias=m.group(7) == "b")  # fmt: skip
 
     def validate(self):
@@ -130,7 +134,7 @@ def _get_kernel_spec(params: LayerNorm2dParams, config: LayerNorm2dConfig, devic
         "SPIO_LN_C": params.c, "SPIO_LN_PIXELS": params.pixels, "SPIO_LN_LPP": lpp,
         "SPIO_LN_THREADS": config.threads, "SPIO_LN_UNROLL": config.unroll,
         "SPIO_LN_HAS_WEIGHT": int(params.has_weight), "SPIO_LN_HAS_BIAS": int(params.has_bias),
-        "SPIO_LN_EPS": f"{params.eps:.9g}f", "SPIO_LN_GRID": grid,
+        "SPIO_LN_EPS": f"{float(params.eps)!r}f", "SPIO_LN_GRID": grid,
     }  # fmt: skip
     return KernelSpec(defines, LaunchParams(grid=grid, block=config.threads), SOURCE,
                       notes={"LPP": lpp, "PASS_PIXELS": pass_pixels})  # fmt: skip
@@ -218,7 +222,7 @@ def _get_bwd_kernel_spec(params: LayerNorm2dParams, config: LayerNorm2dBwdConfig
         "SPIO_LN_C": params.c, "SPIO_LN_PIXELS": params.pixels, "SPIO_LN_LPP": lpp,
         "SPIO_LN_THREADS": config.threads, "SPIO_LN_UNROLL": config.unroll,
         "SPIO_LN_HAS_WEIGHT": int(params.has_weight),
-        "SPIO_LN_EPS": f"{params.eps:.9g}f", "SPIO_LN_GRID": grid,
+        "SPIO_LN_EPS": f"{float(params.eps)!r}f", "SPIO_LN_GRID": grid,
     }  # fmt: skip
     spec = KernelSpec(defines, LaunchParams(grid=grid, block=config.threads), BWD_SOURCE,
                       notes={"LPP": lpp, "PASS_PIXELS": pass_pixels, "GRID": grid})  # fmt: skip

@@ -46,7 +46,7 @@ _PACKAGE_RECORDS = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tun
 ROTATION_BYTES = 600 * 1024 * 1024
 MAX_ROTATION_SETS = 8
 DEFAULT_ON_MISS_CONFIGS = 8
-FINALISTS = 4  # leaders of a sweep that are timed again before one is chosen
+FINALISTS = 6  # leaders of a sweep that are timed again before one is chosen
 
 
 def _on_miss_limit() -> int:

@@ -6,7 +6,7 @@ the ConvNeXt-shaped network.  GPU only."""
 import pytest
 import torch
 
-from convnext_gw8 import ConvNeXtGw8
+from spio_amd.convnext_gw8 import ConvNeXtGw8
 from helpers import to_gpu
 from oracle import conv2d_gw8_oracle as oracle
 from spio_amd.functional import conv2d_gw8
@@ -184,3 +184,27 @@ def test_convnext_shaped_network_with_layernorm_kernels():
     got = got.float().cpu()
     assert float((got - want).abs().max()) < 0.08 * max(1.0, float(want.abs().max()))
     assert torch.equal(got.argmax(dim=1), want.argmax(dim=1))
+
+
+def test_convnext_shaped_network_at_batch_128():
+    """The configuration the benchmark times: batch 128, Conv2dGw8 and LayerNorm2d kernel layers,
+    fp16 autocast, channels_last.  The network treats every image on its own, so the logits of
+    the first 8 images of the batch are compared with the fp32 CPU model run on those 8 images."""
+    from spio_amd.layers import LayerNorm2d
+
+    torch.manual_seed(3)
+    cpu_model = ConvNeXtGw8().eval()
+    images = torch.randn(128, 3, 224, 224, generator=torch.Generator().manual_seed(3)).half()
+    with torch.no_grad():
+        want = cpu_model(images[:8].float())
+    gpu_model = ConvNeXtGw8(make_conv=lambda d: Conv2dGw8(d, d, 3, padding=1, groups=d // 8),
+                            norm2d=lambda d: LayerNorm2d(d, eps=1e-5))  # fmt: skip
+    gpu_model.load_state_dict(cpu_model.state_dict())
+    gpu_model = gpu_model.eval().cuda().to(memory_format=torch.channels_last)
+    with torch.no_grad(), torch.autocast(device_type="cuda", dtype=torch.float16):
+        got = gpu_model(images.cuda().contiguous(memory_format=torch.channels_last))
+    assert got.shape == (128, 1000)
+    got8 = got[:8].float().cpu()
+    assert float((got8 - want).abs().max()) < 0.08 * max(1.0, float(want.abs().max()))
+    assert torch.equal(got8.argmax(dim=1), want.argmax(dim=1))
+    assert torch.isfinite(got).all()

@@ -58,6 +58,31 @@ def test_wgrad_sanity(params):
     run_grad_kernel_test(conv2d_gw8_wgrad_kernel_factory, params)
 
 
+def test_two_tile_heights_and_prefetch_ramp():
+    """Row blocks of two alternating heights (the second half of the grid takes the second height)
+    and the ramped prefetch, forward and data gradient: image heights that are and are not
+    multiples of the pair, a last pair that lies partly outside the image, images side by side,
+    split tiles, a bias, a 5x5 filter, padding that changes the image size."""
+    C = Conv2dGw8Config
+    cases = [
+        (Conv2dGw8Params(n=5, c=64, h=28, w=28, padding=1, has_bias=True),
+         [C(groups=8, block_p=9, block_p2=5, prefetch=4), C(groups=4, block_p=18, block_p2=10, prefetch=12, prefetch_start=3, prefetch_rate=2),
+          C(groups=8, block_p=5, block_p2=9, prefetch=8, block_n=2, split=2, prefetch_start=2, prefetch_rate=3)]),
+        (Conv2dGw8Params(n=3, c=24, h=19, w=20, padding=0, has_bias=False),
+         [C(groups=3, block_p=7, block_p2=4, prefetch=4), C(groups=3, block_p=4, block_p2=1, prefetch=2, xcd_chunk=0),
+          C(groups=3, block_p=16, block_p2=1, prefetch=4, prefetch_start=2, prefetch_rate=1)]),
+        (Conv2dGw8Params(n=2, c=40, h=9, w=9, r=5, s=5, padding=2, has_bias=True),
+         [C(groups=5, block_p=3, block_p2=2, prefetch=2), C(groups=5, block_p=6, block_p2=3, prefetch=4, prefetch_start=2, prefetch_rate=2)]),
+        (Conv2dGw8Params(n=1, c=128, h=64, w=64, padding=7, has_bias=False),
+         [C(groups=8, block_p=20, block_p2=12, prefetch=8, prefetch_start=4, prefetch_rate=2)]),
+        (Conv2dGw8Params(n=4, c=128, h=32, w=32, padding=(2, 0), r=4, s=1, has_bias=True),
+         [C(groups=8, block_p=10, block_p2=7, prefetch=4)]),
+    ]  # fmt: skip
+    for params, configs in cases:
+        run_kernel_test(conv2d_gw8_kernel_factory, params, configs=configs)
+        run_grad_kernel_test(conv2d_gw8_kernel_factory, params, configs=configs, igrad=True)
+
+
 # shapes the fused backward kernel has a configuration for: any padding, odd and even filter
 # sizes (7x7 needs more registers than a wave has and stays with the separate kernels)
 FUSED = [p for p in SANITY if bgrad_is_supported(p) and list(conv2d_gw8_bgrad_kernel_factory.configs(p))] + [

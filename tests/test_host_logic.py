@@ -272,6 +272,26 @@ def test_layernorm_lane_choices():
             assert lpp & (lpp - 1) == 0 and lpp * upl >= c // 8 and cfg.unroll * upl <= 8
 
 
+def test_layernorm_eps_encodes_to_identifier_characters_and_round_trips():
+    """The encoded parameters become part of the kernel's extern "C" symbol: every eps must give
+    identifier characters only, decode back to the same value, and compile."""
+    import re
+
+    from spio_amd.kernels import LayerNorm2dParams, layernorm_2d_bwd_kernel_factory, layernorm_2d_kernel_factory
+
+    assert LayerNorm2dParams(n=2, c=96, h=7, w=7).encode() == "2n_96c_7h_7w_1em06eps_wb"  # recorded names
+    for eps in (1e-3, 1e-4, 0.1, 1.5e-5, 1e-12, 1e-5, 1e-6, 1.0, 2.5, 1e20):
+        params = LayerNorm2dParams(n=2, c=96, h=7, w=7, eps=eps, has_bias=False)
+        name = params.encode()
+        assert re.fullmatch(r"[A-Za-z0-9_]+", name), name
+        assert LayerNorm2dParams.decode(name) == params
+    for factory in (layernorm_2d_kernel_factory, layernorm_2d_bwd_kernel_factory):
+        for eps in (1e-3, 1.0):
+            params = LayerNorm2dParams(n=2, c=96, h=7, w=7, eps=eps)
+            kernel = factory.make_kernel(params, factory.configs(params, ATTR)[0], ATTR)
+            kernel.compile()
+            assert kernel.code
+
 
 def test_fused_backward_works_on_the_larger_of_input_and_output():
     """The fused backward kernel's grid and loads per thread follow the domain both tensors sit in:

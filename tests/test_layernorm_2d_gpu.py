@@ -148,9 +148,11 @@ def test_backward_falls_back_to_torch_operations(monkeypatch):
         torch.testing.assert_close(a, b_, rtol=4e-3, atol=2e-2)
 
 
-def test_layer_and_backward():
+@pytest.mark.parametrize("eps", [1e-6, 1e-3])
+def test_layer_and_backward(eps):
+    """eps = 1e-3 has a decimal point in its shortest form: the kernel's name must still be a symbol."""
     torch.manual_seed(0)
-    layer = LayerNorm2d(96, eps=1e-6).cuda()
+    layer = LayerNorm2d(96, eps=eps).cuda()
     with torch.no_grad():
         layer.weight.copy_(torch.randn(96))
         layer.bias.copy_(torch.randn(96))
@@ -162,7 +164,7 @@ def test_layer_and_backward():
     xr = x.half().float().requires_grad_(True)
     wr = layer.weight.detach().cpu().clone().requires_grad_(True)
     br = layer.bias.detach().cpu().clone().requires_grad_(True)
-    yr = _reference(xr, wr, br, 1e-6)
+    yr = _reference(xr, wr, br, eps)
     yr.backward(dy.half().float())
     torch.testing.assert_close(y.float().cpu(), yr.detach(), rtol=2e-3, atol=4e-3)
     torch.testing.assert_close(xg.grad.float().cpu(), xr.grad, rtol=4e-3, atol=4e-3)
