@@ -631,7 +631,7 @@ def bench_batch_sweep(args, device, full=True):
         act = 2 * n * 64 * 56 * 56
         nsets = rotation_sets(2 * act)
         w, sets = make_buffers(params, 0, nsets, device)
-        iters = 200 if n <= 64 else 60
+        iters = 200
         min_seconds = MIN_TIMED_SECONDS if full else MIN_TIMED_SECONDS / 4
         k_fwd = conv2d_gw8_kernel_factory.get_kernel(params, device)
         fb = Conv2dStats(params, output_names="output").bytes

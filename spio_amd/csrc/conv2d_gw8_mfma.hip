@@ -63,6 +63,9 @@ using namespace spio;
 #ifndef SPIO_BP2
 #define SPIO_BP2 0
 #endif
+#ifndef SPIO_BQ
+#define SPIO_BQ 0
+#endif
 #ifndef SPIO_TS
 #define SPIO_TS 1
 #endif
@@ -112,7 +115,14 @@ constexpr int THREADS = 64 * WAVES;
 constexpr int NS = 2 * ((kR + 1) / 2);  // accumulator row slots
 constexpr int NACC = NS / 2;            // accumulators (pairs of slots) per tile
 constexpr int KB = (kS + 3) / 4;        // MFMA K-steps per source row (4 column taps each)
-constexpr int WPI = DW + kS - 1;        // padded width of one image in LDS
+// Column blocks (SPIO_BQ > 0): a workgroup owns BQ output columns of its rows and stages the
+// BQ + S - 1 source columns they need; the S - 1 extra columns hold the neighbouring blocks'
+// pixels, or zeros at the image's edges (reference: block_q / block_w = block_q + S - 1,
+// spio/kernels/conv2d_gw8_kernel.py:92-108, and the column halo of spio/src/conv2d_gw8.cu:71-91).
+// Rows of any width then fit the LDS ring.  0 = the whole width.
+constexpr int BQ = SPIO_BQ > 0 ? SPIO_BQ : DW;
+constexpr int QBLKS = (DW + BQ - 1) / BQ;
+constexpr int WPI = BQ + kS - 1;        // padded width of one image (block) in LDS
 constexpr int F = NB * WPI;             // flattened pixels of a staged row
 constexpr int WT = (F - kS + 1 + 15) / 16;  // 16-pixel tiles per row
 constexpr int TPW = (WT + TS - 1) / TS;     // tiles per wave
@@ -125,13 +135,13 @@ constexpr int OSTRIDE = GB * 16 + 16;               // bytes per pixel in the ou
 constexpr int OUT_ROW_BYTES = 16 * WT * OSTRIDE;
 constexpr int IN_CELLS = F * GB;
 constexpr int LPT = (IN_CELLS + THREADS - 1) / THREADS;  // source cells per thread per row
-constexpr int OUT_CELLS = NB * DW * GB;
+constexpr int OUT_CELLS = NB * BQ * GB;
 constexpr int SPT = (OUT_CELLS + THREADS - 1) / THREADS;  // stores per thread per row
 constexpr int GBLKS = (kGroups + GB - 1) / GB;
 constexpr int PAIRS = (DH + BP + BP2 - 1) / (BP + BP2);  // (BP, BP2) pairs of row blocks per image
 constexpr int PBLKS = BP2 > 0 ? PAIRS : (DH + BP - 1) / BP;  // row blocks of one height per image
 constexpr int NBLKS = (kN + NB - 1) / NB;
-constexpr int HALF_BLOCKS = GBLKS * PBLKS * NBLKS;  // workgroups per tile height
+constexpr int HALF_BLOCKS = GBLKS * PBLKS * QBLKS * NBLKS;  // workgroups per tile height
 constexpr int NUM_BLOCKS = (BP2 > 0 ? 2 : 1) * HALF_BLOCKS;
 
 // The step loop is unrolled completely: every rotation index and every "is there a row to load
@@ -196,7 +206,7 @@ typedef __attribute__((address_space(3))) unsigned char* lds_bytep;
 template <int ROWS>
 SPIO_DEVICE void conv_rows(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ src,
                            const spio_half* __restrict__ weights, const float* __restrict__ bias,
-                           const lds_u4p ring, const int p0, const int n0, const int cb) {
+                           const lds_u4p ring, const int p0, const int q0, const int n0, const int cb) {
     constexpr int STEPS = ROWS + kR - 1;
     const lds_bytep ostage = (lds_bytep)(ring + NR * RING_ROW_UNITS);
 
@@ -235,7 +245,7 @@ SPIO_DEVICE void conv_rows(spio_uint4* __restrict__ dst, const spio_uint4* __res
             const int g = cell % GB;
             const int f = cell / GB;
             const int img = f / WPI;
-            const int col = f % WPI - EPX;
+            const int col = q0 + f % WPI - EPX;
             in_lds[l] = g * GS + f;
             if (col >= 0 && col < SW && cb * GB + g < kGroups)
                 in_voff[l] = (unsigned)(((img * SH * SW + col) * kGroups + cb * GB + g) * 16);
@@ -321,10 +331,11 @@ SPIO_DEVICE void conv_rows(spio_uint4* __restrict__ dst, const spio_uint4* __res
         out_lds[s] = 0;
         if (cell < OUT_CELLS) {
             const int g = cell % GB;
-            const int q = (cell / GB) % DW;
-            const int img = cell / (GB * DW);
+            const int q = (cell / GB) % BQ;
+            const int img = cell / (GB * BQ);
             out_lds[s] = (img * WPI + q) * OSTRIDE + g * 16;
-            if (cb * GB + g < kGroups) out_voff[s] = (unsigned)(((img * DH * DW + q) * kGroups + cb * GB + g) * 16);
+            if (cb * GB + g < kGroups && q0 + q < DW)
+                out_voff[s] = (unsigned)(((img * DH * DW + q0 + q) * kGroups + cb * GB + g) * 16);
         }
     }
 
@@ -580,18 +591,22 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ dst, const spio_uint4* __restrict__ sr
     // workgroup covers only part of a pixel's 128-byte lines (GB * 16 bytes per pixel), the channel
     // blocks that share those lines go fastest instead: dealt to different XCDs, every one of
     // them would fetch the whole lines from memory (measured: twice the algorithmic reads).
+    // Column blocks go before the row blocks: neighbours share S - 1 columns of every row.
     constexpr bool kSplitLines = GBLKS > 1 && (GB * 16) % 128 != 0;
-    const int pb = kSplitLines ? (b / GBLKS) % PBLKS : b % PBLKS;
-    const int cb = kSplitLines ? b % GBLKS : (b / PBLKS) % GBLKS;
-    const int nb = b / (PBLKS * GBLKS);
+    constexpr int TILES = QBLKS * PBLKS;  // tiles of one image and channel block
+    const int t = kSplitLines ? (b / GBLKS) % TILES : b % TILES;
+    const int cb = kSplitLines ? b % GBLKS : (b / TILES) % GBLKS;
+    const int nb = b / (TILES * GBLKS);
+    const int pb = t / QBLKS;
+    const int q0 = (t % QBLKS) * BQ;
     const int n0 = nb * NB;
     if (BP2 > 0) {
         const int p0 = pb * (BP + BP2);
         if (second)
-            conv_rows<(BP2 > 0 ? BP2 : 1)>(dst, src, weights, bias, ring, p0 + BP, n0, cb);
+            conv_rows<(BP2 > 0 ? BP2 : 1)>(dst, src, weights, bias, ring, p0 + BP, q0, n0, cb);
         else
-            conv_rows<BP>(dst, src, weights, bias, ring, p0, n0, cb);
+            conv_rows<BP>(dst, src, weights, bias, ring, p0, q0, n0, cb);
     } else {
-        conv_rows<BP>(dst, src, weights, bias, ring, pb * BP, n0, cb);
+        conv_rows<BP>(dst, src, weights, bias, ring, pb * BP, q0, n0, cb);
     }
 }

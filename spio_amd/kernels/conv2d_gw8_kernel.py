@@ -35,6 +35,7 @@ DEVICE_LDS_BYTES = 160 * 1024
 MAX_IMAGE_CONFIGS = 10  # whole-image configurations that enter the sweep
 MOVER_WAVES = 4  # data-mover waves of the whole-image kernel where it has any: one per SIMD
 PREFETCH_CHOICES = (2, 4, 8, 10, 12, 16)
+COLUMN_BLOCK_CHOICES = (64, 128, 256)  # output columns per workgroup where rows are tiled
 MAX_GEOMETRIES = 30  # tile geometries that enter the sweep; the best few also try the other cache/XCD policies
 
 
@@ -70,6 +71,9 @@ class Conv2dGw8Config:
             the block_p tiles and the second half the block_p2 tiles.  For grids of two
             workgroups per compute unit, which the device starts as two cohorts of which the
             second trails the first by the first's prefetch burst (0: one height).
+        block_q: row-streaming kernel only: output columns per workgroup (0: the whole width).
+            A workgroup then stages block_q + S - 1 source columns of its rows, so rows of any
+            width fit (reference: block_q and block_w, spio/kernels/conv2d_gw8_kernel.py:92-108).
         prefetch_start, prefetch_rate: row-streaming kernel only: rows requested before the
             first step and per step until the requests run `prefetch` rows ahead
             (prefetch_start = 0: all `prefetch` rows at once).
@@ -89,6 +93,7 @@ class Conv2dGw8Config:
     block_p2: int = 0
     prefetch_start: int = 0
     prefetch_rate: int = 1
+    block_q: int = 0
 
 
 def direction_geometry(params: Conv2dGw8Params, igrad: bool) -> Dict[str, int]:
@@ -106,9 +111,10 @@ def mfma_geometry(params: Conv2dGw8Params, config: Conv2dGw8Config, igrad: bool)
     r, s = params.r, params.s
     gb, bp, nb, ts, pf = config.groups, config.block_p, config.block_n, config.split, config.prefetch
     bp2 = config.block_p2
+    bq = config.block_q or d["DW"]
     ns = 2 * ((r + 1) // 2)
     kb = (s + 3) // 4
-    wpi = d["DW"] + s - 1
+    wpi = bq + s - 1
     f = nb * wpi
     wt = divup(f - s + 1, 16)
     fp = 16 * wt + 4 * kb - 1
@@ -121,13 +127,13 @@ def mfma_geometry(params: Conv2dGw8Params, config: Conv2dGw8Config, igrad: bool)
     d.update(
         NS=ns, NACC=ns // 2, KB=kb, WPI=wpi, F=f, WT=wt, TPW=divup(wt, ts), GS=gs,
         THREADS=threads, LDS_BYTES=lds, LPT=divup(f * gb, threads),
-        SPT=divup(nb * d["DW"] * gb, threads),
+        SPT=divup(nb * bq * gb, threads), BQ=bq, QBLKS=divup(d["DW"], bq),
         GBLKS=divup(params.groups, gb), NBLKS=divup(params.n, nb),
         # two tile heights: PBLKS (block_p, block_p2) pairs per image, one workgroup per tile
         PBLKS=divup(d["DH"], bp + bp2) if bp2 else divup(d["DH"], bp),
         STEPS=max(bp, bp2) + r - 1, UNROLL=ns // gcd(ns, pf) * pf,
     )  # fmt: skip
-    d["NUM_BLOCKS"] = (2 if bp2 else 1) * d["GBLKS"] * d["PBLKS"] * d["NBLKS"]
+    d["NUM_BLOCKS"] = (2 if bp2 else 1) * d["GBLKS"] * d["PBLKS"] * d["QBLKS"] * d["NBLKS"]
     return d
 
 
@@ -254,6 +260,7 @@ def _mfma_config_is_legal(params, config, igrad) -> bool:
         and 0 <= config.prefetch_start <= config.prefetch
         and config.prefetch_start != 1
         and config.prefetch_rate >= 1
+        and 0 <= config.block_q <= g["DW"]
         and g["LDS_BYTES"] <= MAX_LDS_BYTES
         and g["LPT"] <= MAX_LOADS_PER_THREAD
         and g["TPW"] * g["NACC"] <= MAX_ACCUMULATORS
@@ -279,9 +286,9 @@ def _mfma_score(params, config, igrad, num_cus: int) -> float:
     depth x resident workgroups) and, weakly, wasted MFMA columns.
     """
     g = mfma_geometry(params, config, igrad)
-    halo = (config.block_p + params.r - 1) / config.block_p
+    halo = (config.block_p + params.r - 1) / config.block_p * (g["BQ"] + params.s - 1) / g["BQ"]
     traffic = 1.0 + 0.5 * (halo - 1.0)
-    useful = config.block_n * g["DW"]
+    useful = config.block_n * g["BQ"]
     tile_eff = useful / (16.0 * g["WT"])
     group_eff = params.groups / (g["GBLKS"] * config.groups)
     per_cu = _resident_workgroups(g["LDS_BYTES"], g["THREADS"])
@@ -299,7 +306,7 @@ def _mfma_score(params, config, igrad, num_cus: int) -> float:
     # a workgroup that covers only part of a 128-byte line of a pixel shares it with another one
     split_line = 1.0 if (config.groups * 16) % 128 == 0 or config.groups == params.groups else 1.12
     # every row block runs block_p steps, also the last, partly empty one
-    ragged = g["PBLKS"] * (config.block_p + config.block_p2) / g["DH"]
+    ragged = g["PBLKS"] * (config.block_p + config.block_p2) / g["DH"] * g["QBLKS"] * g["BQ"] / g["DW"]
     return traffic * quant * ragged * starve * few_waves * alone * big_block * split_line / (tile_eff ** 0.3 * group_eff)
 
 
@@ -338,18 +345,21 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None, igrad: bool = False)
     G = params.groups
     group_choices = sorted({g for g in (4, 8, 16, G) if g <= min(G, MAX_WAVES)}) or [min(G, MAX_WAVES)]
     row_choices = sorted({bp for bp in (2, 4, 7, 8, 14, 16, 28, 32, 56, d["DH"]) if bp <= d["DH"]})
+    # column blocks for wide rows only: narrower ones fit whole and pay no column halo
+    col_choices = [0] + [bq for bq in COLUMN_BLOCK_CHOICES if d["DW"] >= 2 * bq and d["DW"] > 128]
     found = []
-    for gb in group_choices:
-        for nb in (1, 2, 4, 8):
-            for ts in (1, 2, 4):
-                for bp in row_choices:
-                    steps = bp + params.r - 1
-                    for pf in PREFETCH_CHOICES:
-                        if pf > 2 and pf > steps:
-                            continue
-                        cfg = Conv2dGw8Config(groups=gb, block_p=bp, block_n=nb, split=ts, prefetch=pf)
-                        if _mfma_config_is_legal(params, cfg, igrad):
-                            found.append((_mfma_score(params, cfg, igrad, num_cus), cfg))
+    for bq in col_choices:
+        for gb in group_choices:
+            for nb in (1, 2, 4, 8) if bq == 0 else (1,):
+                for ts in (1, 2, 4):
+                    for bp in row_choices:
+                        steps = bp + params.r - 1
+                        for pf in PREFETCH_CHOICES:
+                            if pf > 2 and pf > steps:
+                                continue
+                            cfg = Conv2dGw8Config(groups=gb, block_p=bp, block_n=nb, split=ts, prefetch=pf, block_q=bq)
+                            if _mfma_config_is_legal(params, cfg, igrad):
+                                found.append((_mfma_score(params, cfg, igrad, num_cus), cfg))
     found.sort(key=lambda sc: sc[0])
     configs = [cfg for _, cfg in found[:MAX_GEOMETRIES]]
     # the memory-system policies, which the score cannot rank: halo rows with or without the
@@ -425,6 +435,8 @@ def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8Config, _device_a
         defines["SPIO_PF0"] = config.prefetch_start
     if config.prefetch_rate != 1:
         defines["SPIO_PF_RATE"] = config.prefetch_rate
+    if config.block_q:
+        defines["SPIO_BQ"] = config.block_q
     return KernelSpec(
         defines, LaunchParams(grid=g["NUM_BLOCKS"], block=g["THREADS"]), MFMA_SOURCE, notes=g
     )

@@ -83,6 +83,32 @@ def test_two_tile_heights_and_prefetch_ramp():
         run_grad_kernel_test(conv2d_gw8_kernel_factory, params, configs=configs, igrad=True)
 
 
+def test_column_blocks():
+    """Workgroups that own a block of output columns (block_q) and stage block_q + S - 1 source
+    columns: widths that are and are not multiples of the block, blocks wider than what is left
+    at the right edge, 5x5 and even filters (column halo of 4 and 3), padding 0 and padding
+    larger than the halo, together with two tile heights; forward and data gradient."""
+    C = Conv2dGw8Config
+    cases = [
+        (Conv2dGw8Params(n=3, c=24, h=9, w=150, padding=1, has_bias=True),
+         [C(groups=3, block_p=4, block_q=64, prefetch=4), C(groups=3, block_p=9, block_q=32, prefetch=2, split=2),
+          C(groups=3, block_p=3, block_p2=1, block_q=128, prefetch=4)]),
+        (Conv2dGw8Params(n=2, c=16, h=7, w=100, r=5, s=5, padding=2, has_bias=False),
+         [C(groups=2, block_p=7, block_q=64, prefetch=4), C(groups=2, block_p=2, block_q=16, prefetch=2)]),
+        (Conv2dGw8Params(n=2, c=16, h=6, w=77, r=2, s=4, padding=(0, 3), has_bias=True),
+         [C(groups=2, block_p=3, block_q=32, prefetch=2), C(groups=1, block_p=5, block_q=48, prefetch=4)]),
+        (Conv2dGw8Params(n=2, c=32, h=10, w=70, padding=0, has_bias=False),
+         [C(groups=4, block_p=4, block_q=32, prefetch=4)]),
+        (Conv2dGw8Params(n=4, c=32, h=64, w=512, padding=1, has_bias=False),
+         [C(groups=4, block_p=8, block_q=64, prefetch=8, split=2), C(groups=4, block_p=16, block_q=128, prefetch=4)]),
+        (Conv2dGw8Params(n=2, c=64, h=20, w=1024, padding=1, has_bias=True),
+         [C(groups=8, block_p=10, block_q=128, prefetch=8), C(groups=4, block_p=7, block_q=256, prefetch=4, split=2)]),
+    ]  # fmt: skip
+    for params, configs in cases:
+        run_kernel_test(conv2d_gw8_kernel_factory, params, configs=configs)
+        run_grad_kernel_test(conv2d_gw8_kernel_factory, params, configs=configs, igrad=True)
+
+
 # shapes the fused backward kernel has a configuration for: any padding, odd and even filter
 # sizes (7x7 needs more registers than a wave has and stays with the separate kernels)
 FUSED = [p for p in SANITY if bgrad_is_supported(p) and list(conv2d_gw8_bgrad_kernel_factory.configs(p))] + [
