@@ -57,6 +57,9 @@ using namespace spio;
 #ifndef SPIO_PF
 #define SPIO_PF 2
 #endif
+#ifndef SPIO_BQ
+#define SPIO_BQ 0
+#endif
 #ifndef SPIO_TS
 #define SPIO_TS 1
 #endif
@@ -102,9 +105,20 @@ constexpr int S2 = 2 * ((kS + 1) / 2);
 constexpr int NBLK = S2 / 2;          // column-tap pairs
 constexpr int ND = kR + 1;            // values of delta
 constexpr int NPAIR = kR / 2 + 1;     // aligned dy row pairs one x row meets
-constexpr int WPI = DW + kS - 1;      // padded width of one image
+// Column blocks (SPIO_BQ > 0): a workgroup owns BQ columns (of dx, and of dy for the weight
+// gradient) and stages BQ + S - 1 columns of x and of dy: the extra columns hold the neighbouring
+// blocks' pixels (the data gradient of the block's edge columns needs the neighbours' dy, the
+// weight gradient the neighbours' x), or zeros at the image's edges.  The weight gradient reads dy
+// in 32-pixel chunks from the block's first column on, so BQ is a multiple of 32: a chunk that
+// reached into the right-hand extra columns would count the neighbour's dy a second time.
+// 0 = the whole width.
+constexpr bool kColBlocks = SPIO_BQ > 0;
+constexpr int BQ = kColBlocks ? SPIO_BQ : DW;
+constexpr int QBLKS = (DW + BQ - 1) / BQ;
+static_assert(!kColBlocks || (NB == 1 && BQ % 32 == 0), "column blocks: one image per row, a multiple of 32 columns");
+constexpr int WPI = BQ + kS - 1;      // padded width of one image (block)
 constexpr int F = NB * WPI;           // flattened pixels of a staged row
-constexpr int KSPAN = (NB - 1) * WPI + DW;
+constexpr int KSPAN = (NB - 1) * WPI + BQ;
 constexpr int KC = (KSPAN + 31) / 32;     // 32-pixel chunks
 constexpr int CPW = (KC + TS - 1) / TS;   // chunks per wave
 // ---- data gradient ----
@@ -135,12 +149,16 @@ constexpr int OSTRIDE = GB * 16 + 16;        // bytes per pixel in the dx output
 constexpr int OUT_ROW_BYTES = 16 * WT * OSTRIDE;
 constexpr int X_CELLS = F * GB;
 constexpr int LPTX = (X_CELLS + THREADS - 1) / THREADS;
-constexpr int D_CELLS = NB * DW * GB;
-constexpr int LPTD = (D_CELLS + THREADS - 1) / THREADS;  // dy loads = dx stores per thread per row
+// dy cells a workgroup loads per row: the real columns of whole rows (the halo stays zero), all
+// BQ + S - 1 columns of a column block
+constexpr int D_CELLS = kColBlocks ? F * GB : NB * DW * GB;
+constexpr int LPTD = (D_CELLS + THREADS - 1) / THREADS;  // dy loads per thread per row
+constexpr int O_CELLS = NB * BQ * GB;
+constexpr int LPTO = (O_CELLS + THREADS - 1) / THREADS;  // dx stores per thread per row
 constexpr int GBLKS = (kGroups + GB - 1) / GB;
 constexpr int NBLKS = (kN + NB * ITERS - 1) / (NB * ITERS);
 constexpr int PBLKS = (DH + BH - 1) / BH;
-constexpr int NUM_BLOCKS = GBLKS * PBLKS * NBLKS;
+constexpr int NUM_BLOCKS = GBLKS * PBLKS * QBLKS * NBLKS;
 // steps: dy rows p0-PB .. p0+BH-1+PT, then PB more for the last x rows.  The bias sum takes a dy
 // row pair one step after its first row was staged, so a one-row filter needs one more step
 // when the sum is wanted.
@@ -239,9 +257,13 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
     // blocks that share those lines go fastest instead: dealt to different XCDs, every one of
     // them would fetch the whole lines from memory (measured: twice the algorithmic reads).
     constexpr bool kSplitLines = GBLKS > 1 && (GB * 16) % 128 != 0;
-    const int pb = kSplitLines ? (b / GBLKS) % PBLKS : b % PBLKS;
-    const int cb = kSplitLines ? b % GBLKS : (b / PBLKS) % GBLKS;
-    const int nbk = b / (PBLKS * GBLKS);
+    // Column blocks go before the row blocks: neighbours share S - 1 columns of every row.
+    constexpr int TILES = QBLKS * PBLKS;
+    const int tile = kSplitLines ? (b / GBLKS) % TILES : b % TILES;
+    const int cb = kSplitLines ? b % GBLKS : (b / TILES) % GBLKS;
+    const int nbk = b / (TILES * GBLKS);
+    const int pb = tile / QBLKS;
+    const int q0 = (tile % QBLKS) * BQ;
     const int p0 = pb * BH;
     const int bh_eff = imin(BH, DH - p0);  // rows this block owns
     // first and last row (of the domain) the block needs: of x for the weight gradient of its dy
@@ -329,7 +351,7 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                 const int g = cell % GB;
                 const int f = cell / GB;
                 const int img = f / WPI;
-                const int col = f % WPI - PL - XOX;  // column of x
+                const int col = q0 + f % WPI - PL - XOX;  // column of x
                 x_lds[l] = g * GSX + f;
                 if (col >= 0 && col < kW && cb * GB + g < kGroups)
                     x_voff[l] = (unsigned)(((img * kH * kW + col) * kGroups + cb * GB + g) * 16);
@@ -337,26 +359,36 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
         }
         // dy cells, and the dx cells of the same (image, domain column, group): where dy and x have
         // the same size, the same offset
-        unsigned d_voff[LPTD], o_voff[LPTD];
-        int d_lds[LPTD], o_lds[LPTD];
+        unsigned d_voff[LPTD], o_voff[LPTO];
+        int d_lds[LPTD], o_lds[LPTO];
 #pragma unroll
         for (int l = 0; l < LPTD; ++l) {
             const int cell = tid + THREADS * l;
             d_voff[l] = OOB;
-            o_voff[l] = OOB;
             d_lds[l] = DDUMP;
-            o_lds[l] = 0;
             if (cell < D_CELLS) {
                 const int g = cell % GB;
-                const int q = (cell / GB) % DW;
-                const int img = cell / (GB * DW);
-                d_lds[l] = g * GSD + img * WPI + q + PR;
-                o_lds[l] = (img * WPI + q) * OSTRIDE + g * 16;
+                // whole rows: the cells are the real columns; column blocks: every staged column
+                const int q = kColBlocks ? q0 + (cell / GB) % WPI - PR : (cell / GB) % DW;  // domain column
+                const int img = kColBlocks ? 0 : cell / (GB * DW);
+                d_lds[l] = g * GSD + (kColBlocks ? cell / GB : img * WPI + q + PR);
                 const int qd = q - DOX;  // column of dy
-                const int wx = q - XOX;  // column of dx
                 if (qd >= 0 && qd < kQ && cb * GB + g < kGroups)
                     d_voff[l] = (unsigned)(((img * kP * kQ + qd) * kGroups + cb * GB + g) * 16);
-                if (wx >= 0 && wx < kW && cb * GB + g < kGroups)
+            }
+        }
+#pragma unroll
+        for (int l = 0; l < LPTO; ++l) {
+            const int cell = tid + THREADS * l;
+            o_voff[l] = OOB;
+            o_lds[l] = 0;
+            if (cell < O_CELLS) {
+                const int g = cell % GB;
+                const int q = (cell / GB) % BQ;
+                const int img = cell / (GB * BQ);
+                o_lds[l] = (img * WPI + q) * OSTRIDE + g * 16;
+                const int wx = q0 + q - XOX;  // column of dx
+                if (q0 + q < DW && wx >= 0 && wx < kW && cb * GB + g < kGroups)
                     o_voff[l] = (unsigned)(((img * kH * kW + wx) * kGroups + cb * GB + g) * 16);
             }
         }
@@ -462,7 +494,7 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
             // (seen on gfx950 as stray values in the first two channels of some pixels).
             const unsigned row_off = (unsigned)(imin(imax(h - XOY, 0), kH - 1) * X_ROW_BYTES);
 #pragma unroll
-            for (int l = 0; l < LPTD; ++l) {
+            for (int l = 0; l < LPTO; ++l) {
                 Pack16 v;
                 v.u = *reinterpret_cast<const spio_uint4*>(ostage + obuf * OUT_ROW_BYTES + o_lds[l]);
                 __builtin_amdgcn_raw_buffer_store_b128(v.i, rs, (int)(o_voff[l] + row_off), 0, AUX_NT);

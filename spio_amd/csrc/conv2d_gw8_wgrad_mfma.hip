@@ -57,6 +57,9 @@ using namespace spio;
 #ifndef SPIO_PARTIALS
 #define SPIO_PARTIALS 0
 #endif
+#ifndef SPIO_BQ
+#define SPIO_BQ 0
+#endif
 #ifndef SPIO_TS
 #define SPIO_TS 1
 #endif
@@ -82,9 +85,14 @@ constexpr int RB = SPIO_RB;  // x rows (and dy rows) per step: 1 or 2
 constexpr int S2 = 2 * ((kS + 1) / 2);
 constexpr int NBLK = S2 / 2;   // column-tap pairs
 constexpr int ND = kR + 1;     // values of delta
-constexpr int WPI = kQ + kS - 1;  // padded width of one image (= W + 2*px)
+// Column blocks (SPIO_BQ > 0): a workgroup sums over BQ columns of dy and the BQ + S - 1 columns
+// of x opposite them, so rows of any width fit the rings (the reference tiles the width with a
+// fixed block of 8 columns, spio/kernels/conv2d_gw8_wgrad_kernel.py:40).  0 = the whole width.
+constexpr int BQ = SPIO_BQ > 0 ? SPIO_BQ : kQ;
+constexpr int QBLKS = (kQ + BQ - 1) / BQ;
+constexpr int WPI = BQ + kS - 1;  // padded width of one image (block): W + 2*px for whole rows
 constexpr int F = NB * WPI;
-constexpr int KSPAN = (NB - 1) * WPI + kQ;  // flattened pixels that carry dy
+constexpr int KSPAN = (NB - 1) * WPI + BQ;  // flattened pixels that carry dy
 constexpr int KC = (KSPAN + 31) / 32;       // 32-pixel chunks
 constexpr int FPX = 32 * KC + S2 - 1;
 constexpr int GSX = FPX + ((9 - FPX % 16) + 16) % 16;  // x group stride (pixels), = 9 mod 16
@@ -102,12 +110,12 @@ constexpr int XROW_UNITS = GB * GSX;
 constexpr int DROW_UNITS = GB * GSD + ((4 - (GB * GSD) % 16) + 16) % 16;
 constexpr int X_CELLS = F * GB;
 constexpr int LPTX = (X_CELLS + THREADS - 1) / THREADS;
-constexpr int D_CELLS = NB * kQ * GB;
+constexpr int D_CELLS = NB * BQ * GB;
 constexpr int LPTD = (D_CELLS + THREADS - 1) / THREADS;
 constexpr int GBLKS = (kGroups + GB - 1) / GB;
 constexpr int PBLKS = (kP + BH - 1) / BH;
 constexpr int NBLKS = (kN + NB * ITERS - 1) / (NB * ITERS);
-constexpr int NUM_BLOCKS = GBLKS * PBLKS * NBLKS;
+constexpr int NUM_BLOCKS = GBLKS * PBLKS * QBLKS * NBLKS;
 constexpr bool kDbias = SPIO_HAS_BIAS != 0;  // also sum grad_output per channel (grad_bias)
 // x rows a workgroup streams.  The bias sum takes a grad_output row pair one step after its
 // first row was staged, so a one-row filter needs one more step when the sum is wanted.
@@ -174,9 +182,11 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
 
     int b = block_id();
     if (NUM_BLOCKS % 8 == 0) b = (b & 7) * (NUM_BLOCKS / 8) + (b >> 3);
-    const int pb = b % PBLKS;
-    const int cb = (b / PBLKS) % GBLKS;
-    const int nbk = b / (PBLKS * GBLKS);
+    const int qb = b % QBLKS;  // column blocks fastest: neighbours share S - 1 columns of x
+    const int q0 = qb * BQ;
+    const int pb = (b / QBLKS) % PBLKS;
+    const int cb = (b / (QBLKS * PBLKS)) % GBLKS;
+    const int nbk = b / (QBLKS * PBLKS * GBLKS);
     const int p0 = pb * BH;
     const int bh_eff = imin(BH, kP - p0);  // dy rows that exist in this block
     const int gglob = cb * GB + wg;
@@ -229,7 +239,7 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
                 const int g = cell % GB;
                 const int f = cell / GB;
                 const int img = f / WPI;
-                const int col = f % WPI - kPadX;
+                const int col = q0 + f % WPI - kPadX;
                 x_lds[l] = g * GSX + f;
                 if (col >= 0 && col < kW && n0 + img < kN && cb * GB + g < kGroups) {
                     x_off[l] = ((n0 + img) * kH * kW + col) * kGroups + cb * GB + g;
@@ -248,11 +258,11 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
             d_lds[l] = -1;
             if (cell < D_CELLS) {
                 const int g = cell % GB;
-                const int q = (cell / GB) % kQ;
-                const int img = cell / (GB * kQ);
+                const int q = (cell / GB) % BQ;
+                const int img = cell / (GB * BQ);
                 d_lds[l] = g * GSD + img * WPI + q;
-                if (n0 + img < kN && cb * GB + g < kGroups) {
-                    d_off[l] = ((n0 + img) * kP * kQ + q) * kGroups + cb * GB + g;
+                if (q0 + q < kQ && n0 + img < kN && cb * GB + g < kGroups) {
+                    d_off[l] = ((n0 + img) * kP * kQ + q0 + q) * kGroups + cb * GB + g;
                     d_ok[l] = true;
                 }
             }
@@ -443,7 +453,7 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
 #if SPIO_PARTIALS
         // this wave's slice of the workgroup's partial block: [r][tap pair][e][32 lanes], so that
         // every store instruction writes 128 contiguous bytes
-        float* out = grad_weight + (((long long)(nbk * PBLKS + pb) * GBLKS + cb) * GB + wg) * PART_WAVE_FLOATS;
+        float* out = grad_weight + (((long long)((nbk * PBLKS + pb) * QBLKS + qb) * GBLKS + cb) * GB + wg) * PART_WAVE_FLOATS;
 #else
         float* out = grad_weight;
 #endif
@@ -633,7 +643,7 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
 extern "C" __global__ void SPIO_LAUNCH_BOUNDS(256)
 SPIO_CONCAT(SPIO_KERNEL_NAME, _reduce)(float* __restrict__ grad_weight, const spio_float4* __restrict__ partials) {
     constexpr int BLOCK_F4 = GB * PART_WAVE_FLOATS / 4;  // float4 columns of one partial block
-    constexpr int NPART = NBLKS * PBLKS;
+    constexpr int NPART = NBLKS * PBLKS * QBLKS;
     constexpr int COLS = 32;
     constexpr int SLICES = 256 / COLS;
     constexpr int UN = 4;

@@ -53,6 +53,9 @@ class Conv2dGw8BgradConfig:
             cache policy (the second reader can hit in L2), the others with the non-temporal hint.
         xcd_chunk: consecutive tiles that go to the same XCD before the next run goes to the next
             one; 0 = one contiguous range of tiles per XCD.
+        block_q: columns per workgroup (0: the whole width; else a multiple of 32 with
+            block_n = 1).  The workgroup stages block_q + S - 1 columns of x and of grad_output, so
+            rows of any width fit.
     """
 
     groups: int = 4
@@ -63,6 +66,7 @@ class Conv2dGw8BgradConfig:
     split: int = 1
     halo_cached: int = 1
     xcd_chunk: int = 4
+    block_q: int = 0
 
 
 def bgrad_is_supported(params: Conv2dGw8Params) -> bool:
@@ -100,9 +104,10 @@ def bgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig) -> Dic
     bh = config.block_h or dh
     s2 = 2 * ((s + 1) // 2)
     nblk = s2 // 2
-    wpi = dw + s - 1
+    bq = config.block_q or dw
+    wpi = bq + s - 1
     f = nb * wpi
-    kspan = (nb - 1) * wpi + dw
+    kspan = (nb - 1) * wpi + bq
     kc = divup(kspan, 32)
     cpw = divup(kc, ts)
     ns = 2 * ((r + 1) // 2)
@@ -124,7 +129,7 @@ def bgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig) -> Dic
     publish_bytes = (gb * ts * rch * nblk * 128 + gb * (ts - 1) * nblk * 128 + gb * r * s * 64
                      + (gb * ts * 8 if params.has_bias else 0)) * 4  # fmt: skip
     lptx = divup(f * gb, threads)
-    lptd = divup(nb * dw * gb, threads)
+    lptd = divup((f if config.block_q else nb * dw) * gb, threads)  # grad_output loads per row
     registers = (
         4 * ((r + 1) * nblk + 1)  # weight-gradient accumulators (+ bias)
         + 4 * tpw * (ns // 2)  # data-gradient accumulators
@@ -138,9 +143,10 @@ def bgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig) -> Dic
         LPTX=lptx, LPTD=lptd, REGISTERS=registers,
         STEPS=bh + pb + r - 1 + (1 if params.has_bias and r == 1 else 0),
         BH=bh, GBLKS=divup(params.groups, gb), PBLKS=divup(dh, bh), NBLKS=divup(params.n, nb * iters),
-        PIXEL_EFF=(nb * dw) / (32.0 * kc),
+        BQ=bq, QBLKS=divup(dw, bq),
+        PIXEL_EFF=(nb * bq) / (32.0 * kc),
     )  # fmt: skip
-    g["NUM_BLOCKS"] = g["GBLKS"] * g["PBLKS"] * g["NBLKS"]
+    g["NUM_BLOCKS"] = g["GBLKS"] * g["PBLKS"] * g["QBLKS"] * g["NBLKS"]
     return g
 
 
@@ -152,6 +158,9 @@ def _config_is_legal(params, config) -> bool:
         config.groups * config.split <= MAX_WAVES
         and config.split <= min(g["KC"], g["WT"])
         and 0 <= config.block_h <= bgrad_domain(params)[0]
+        and 0 <= config.block_q <= bgrad_domain(params)[1]
+        and (config.block_q == 0 or (config.block_q % 32 == 0 and config.block_n == 1))
+        and g["LPTD"] <= MAX_LOADS_PER_THREAD
         and config.block_n * config.block_n_iters <= max(params.n, 1)
         and g["LDS_BYTES"] <= MAX_LDS_BYTES
         and g["LPTX"] <= MAX_LOADS_PER_THREAD
@@ -200,17 +209,20 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None) -> List[Conv2dGw8Bgr
     if wpi < 32:
         best = max(chunk_fill(nb) for nb in image_counts)
         image_counts += [nb for nb in (3, 5, 6, 7) if chunk_fill(nb) > best + 0.05]
+    # column blocks for wide rows only: narrower ones fit whole
+    col_choices = [0] + [bq for bq in (64, 128) if dw >= 2 * bq and dw > 128]
     configs = []
     for bh in row_choices:
         geometries = []
-        for gb in group_choices:
-            for nb in image_counts:
-                for iters in (1, 2, 4):
-                    for ts in (1, 2):
-                        cfg = Conv2dGw8BgradConfig(groups=gb, block_h=bh, block_n=nb, block_n_iters=iters,
-                                                   prefetch=4, split=ts)  # fmt: skip
-                        if _config_is_legal(params, cfg):
-                            geometries.append((_score(params, cfg, num_cus), cfg))
+        for bq in col_choices:
+            for gb in group_choices:
+                for nb in image_counts if bq == 0 else (1,):
+                    for iters in (1, 2, 4):
+                        for ts in (1, 2):
+                            cfg = Conv2dGw8BgradConfig(groups=gb, block_h=bh, block_n=nb, block_n_iters=iters,
+                                                       prefetch=4, split=ts, block_q=bq)  # fmt: skip
+                            if _config_is_legal(params, cfg):
+                                geometries.append((_score(params, cfg, num_cus), cfg))
         geometries.sort(key=lambda sc: sc[0])
         configs += [cfg for _, cfg in geometries[:GEOMETRIES_PER_HEIGHT]]
     # a shallower and a deeper pipeline for the first few: the shallow one wins where rows are short
@@ -232,6 +244,8 @@ def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig, _dev
                    SPIO_PF=config.prefetch, SPIO_TS=config.split,
                    SPIO_HALO_CACHED=config.halo_cached, SPIO_XCD_CHUNK=config.xcd_chunk,
                    SPIO_HAS_BIAS=int(params.has_bias))  # fmt: skip
+    if config.block_q:
+        defines["SPIO_BQ"] = config.block_q
     return KernelSpec(defines, LaunchParams(grid=g["NUM_BLOCKS"], block=g["THREADS"]), SOURCE, notes=g)
 
 

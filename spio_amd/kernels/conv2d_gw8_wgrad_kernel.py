@@ -53,6 +53,8 @@ class Conv2dGw8WgradConfig:
         two_stage: 1 = workgroups store partial sums to a workspace and a second kernel
             reduces them; 0 = workgroups add into grad_weight with fp32 atomics.
         variant: "mfma" (row-streaming MFMA kernel) or "direct" (any shape).
+        block_q: grad_output columns per workgroup (0: the whole width); the workgroup stages
+            block_q + S - 1 columns of x opposite them, so rows of any width fit.
     """
 
     groups: int = 8
@@ -65,6 +67,7 @@ class Conv2dGw8WgradConfig:
     two_stage: int = 0
     split: int = 1
     rows: int = 1
+    block_q: int = 0
 
 
 def wgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig) -> Dict[str, int]:
@@ -72,9 +75,10 @@ def wgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig) -> Dic
     r, s = params.r, params.s
     gb, bh, nb, iters, ts = config.groups, config.block_h, config.block_n, config.block_n_iters, config.split
     s2 = 2 * ((s + 1) // 2)
-    wpi = params.q + s - 1
+    bq = config.block_q or params.q
+    wpi = bq + s - 1
     f = nb * wpi
-    kspan = (nb - 1) * wpi + params.q
+    kspan = (nb - 1) * wpi + bq
     kc = divup(kspan, 32)
     fpx = 32 * kc + s2 - 1
     gsx = fpx + ((9 - fpx % 16) + 16) % 16
@@ -94,13 +98,14 @@ def wgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig) -> Dic
     g = dict(
         NBLK=s2 // 2, ND=r + 1, WPI=wpi, F=f, KC=kc, GSX=gsx, GSD=gsd, NRD=nrd, THREADS=threads,
         LDS_BYTES=max(lds_rings, lds_scratch), RING_BYTES=lds_rings, SCRATCH_BYTES=lds_scratch,
-        LPTX=divup(f * gb, threads), LPTD=divup(nb * params.q * gb, threads),
+        LPTX=divup(f * gb, threads), LPTD=divup(nb * bq * gb, threads),
+        BQ=bq, QBLKS=divup(params.q, bq),
         GBLKS=divup(params.groups, gb), PBLKS=divup(params.p, bh),
         NBLKS=divup(params.n, nb * iters),
         STEPS=divup(bh + (2 if params.has_bias and r == 1 else r) - 1, rb),
-        PIXEL_EFF=kspan and (nb * params.q) / (32.0 * kc),
+        PIXEL_EFF=kspan and (nb * bq) / (32.0 * kc),
     )  # fmt: skip
-    g["NUM_BLOCKS"] = g["GBLKS"] * g["PBLKS"] * g["NBLKS"]
+    g["NUM_BLOCKS"] = g["GBLKS"] * g["PBLKS"] * g["QBLKS"] * g["NBLKS"]
     return g
 
 
@@ -117,6 +122,7 @@ def _mfma_config_is_legal(params, config) -> bool:
         and config.prefetch >= 2
         and config.prefetch % 2 == 0
         and config.rows in (1, 2)
+        and 0 <= config.block_q <= params.q
         and (g["LPTX"] + g["LPTD"]) * config.prefetch * config.rows <= 32
     )
 
@@ -125,7 +131,7 @@ def _mfma_score(params, config, num_cus) -> float:
     """Rough relative cost used only to order (and cap) the sweep; lower is better."""
     g = wgrad_geometry(params, config)
     halo = (config.block_h + params.r - 1) / config.block_h
-    traffic = 1.0 + 0.5 * (halo - 1.0)
+    traffic = 1.0 + 0.5 * (halo - 1.0) + 0.25 * (params.s - 1) / g["BQ"]
     group_eff = params.groups / (g["GBLKS"] * config.groups)
     # compute units idle in the last round of workgroups
     quant = divup(g["NUM_BLOCKS"], num_cus) * num_cus / g["NUM_BLOCKS"]
@@ -168,17 +174,20 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None) -> List[Conv2dGw8Wgr
         image_counts += [nb for nb in (3, 5, 6, 7) if chunk_fill(nb) > best + 0.05]
     # Rank the tile geometries first and keep the best few; each of them is then tried with the
     # pipeline variants (prefetch distance, rows per step), which the score cannot tell apart.
+    # column blocks for wide rows only: narrower ones fit whole
+    col_choices = [0] + [bq for bq in (64, 128, 256) if params.q >= 2 * bq and params.q > 128]
     geometries = []
-    for gb in group_choices:
-        for nb in image_counts:
-            for iters in (1, 2, 4, 8):
-                for bh in row_choices:
-                    for two_stage in (0, 1):
-                        for ts in (1, 2):
-                            cfg = Conv2dGw8WgradConfig(groups=gb, block_h=bh, block_n=nb, block_n_iters=iters,
-                                                       prefetch=2, two_stage=two_stage, split=ts)  # fmt: skip
-                            if _mfma_config_is_legal(params, cfg):
-                                geometries.append((_mfma_score(params, cfg, num_cus), cfg))
+    for bq in col_choices:
+        for gb in group_choices:
+            for nb in image_counts if bq == 0 else (1,):
+                for iters in (1, 2, 4, 8):
+                    for bh in row_choices:
+                        for two_stage in (0, 1):
+                            for ts in (1, 2):
+                                cfg = Conv2dGw8WgradConfig(groups=gb, block_h=bh, block_n=nb, block_n_iters=iters,
+                                                           prefetch=2, two_stage=two_stage, split=ts, block_q=bq)  # fmt: skip
+                                if _mfma_config_is_legal(params, cfg):
+                                    geometries.append((_mfma_score(params, cfg, num_cus), cfg))
     geometries.sort(key=lambda sc: sc[0])
     configs = []
     for _, base in geometries[:MAX_GEOMETRIES]:
@@ -213,9 +222,11 @@ def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig, _dev
     defines.update(SPIO_GB=config.groups, SPIO_BH=config.block_h, SPIO_NB=config.block_n,
                    SPIO_ITERS=config.block_n_iters, SPIO_PF=config.prefetch,
                    SPIO_TS=config.split, SPIO_RB=config.rows)  # fmt: skip
+    if config.block_q:
+        defines["SPIO_BQ"] = config.block_q
     spec = KernelSpec(defines, LaunchParams(grid=g["NUM_BLOCKS"], block=g["THREADS"]), MFMA_SOURCE, notes=g)
     if config.two_stage:
-        num_partials = g["NBLKS"] * g["PBLKS"]
+        num_partials = g["NBLKS"] * g["PBLKS"] * g["QBLKS"]
         # float4 columns of the partial blocks of one (image block, row block): per wave
         # [r][tap pair][4][32 lanes] floats
         cols = g["GBLKS"] * config.groups * params.r * g["NBLK"] * 32

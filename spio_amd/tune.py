@@ -22,6 +22,12 @@ BENCH_SHAPES = [
     "128n_128c_28h_28w_1py_1px_3r_3s_nb",
     "256n_256c_14h_14w_3py_3px_7r_7s_nb",
 ]
+# rows wider than the LDS rings hold whole: the kernels tile them into column blocks
+WIDE_SHAPES = [
+    "16n_64c_128h_512w_1py_1px_3r_3s_nb",
+    "8n_64c_64h_1024w_1py_1px_3r_3s_nb",
+    "32n_64c_224h_224w_1py_1px_3r_3s_nb",
+]
 SWEEP_BATCHES = [1, 2, 4, 8, 16, 32, 64, 128, 256, 512]
 NETWORK_SHAPES = [
     "128n_96c_56h_56w_1py_1px_3r_3s_b",
@@ -190,7 +196,7 @@ class _NullContext:
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("shapes", nargs="*", help="shapes in Conv2dGw8Params.encode() form")
-    ap.add_argument("--shapes", dest="preset", choices=["bench", "batch-sweep", "network", "all"])
+    ap.add_argument("--shapes", dest="preset", choices=["bench", "batch-sweep", "network", "wide", "all"])
     ap.add_argument("--directions", default="fprop,dgrad,wgrad,bgrad",
                     help="bgrad = the fused data+weight gradient kernel")
     ap.add_argument("--iters", type=int, default=30)
@@ -219,6 +225,8 @@ def main(argv=None):
         shapes += [f"{n}n_64c_56h_56w_1py_1px_3r_3s_nb" for n in SWEEP_BATCHES]
     if args.preset in ("network", "all"):
         shapes += NETWORK_SHAPES
+    if args.preset in ("wide", "all"):
+        shapes += WIDE_SHAPES
     if not shapes:
         ap.error("no shapes given")
     if not torch.cuda.is_available():

@@ -13,6 +13,7 @@ from spio_amd.kernels import (
     Conv2dGw8BgradConfig,
     Conv2dGw8Config,
     Conv2dGw8Params,
+    Conv2dGw8WgradConfig,
     bgrad_is_supported,
     conv2d_gw8_bgrad_kernel_factory,
     conv2d_gw8_kernel_factory,
@@ -107,6 +108,38 @@ def test_column_blocks():
     for params, configs in cases:
         run_kernel_test(conv2d_gw8_kernel_factory, params, configs=configs)
         run_grad_kernel_test(conv2d_gw8_kernel_factory, params, configs=configs, igrad=True)
+
+
+def test_column_blocks_weight_gradient_and_fused_backward():
+    """Column blocks in the weight-gradient kernel (atomics and two-stage) and in the fused
+    backward kernel (blocks of 32k columns): each grad_output column is counted by exactly one
+    workgroup, the x columns opposite a block's edges come from the neighbouring blocks."""
+    W = Conv2dGw8WgradConfig
+    B = Conv2dGw8BgradConfig
+    cases = [
+        (Conv2dGw8Params(n=3, c=24, h=9, w=150, padding=1, has_bias=True),
+         [W(groups=3, block_h=4, block_q=64, prefetch=2), W(groups=3, block_h=9, block_q=64, prefetch=2, split=2, two_stage=1),
+          W(groups=3, block_h=8, block_q=48, prefetch=2, rows=2)],
+         [B(groups=3, block_h=0, block_q=64, prefetch=2), B(groups=3, block_h=7, block_q=64, prefetch=4, split=2), B(groups=3, block_h=4, block_q=32, prefetch=2)]),
+        (Conv2dGw8Params(n=2, c=16, h=7, w=100, r=5, s=5, padding=2, has_bias=False),
+         [W(groups=2, block_h=7, block_q=64, prefetch=2), W(groups=2, block_h=4, block_q=16, prefetch=2, two_stage=1)],
+         [B(groups=2, block_h=0, block_q=32, prefetch=2), B(groups=2, block_h=3, block_q=64, prefetch=2, split=2)]),
+        (Conv2dGw8Params(n=2, c=16, h=6, w=77, r=2, s=4, padding=(0, 3), has_bias=True),
+         [W(groups=2, block_h=4, block_q=32, prefetch=2)],
+         [B(groups=2, block_h=0, block_q=32, prefetch=2)]),
+        (Conv2dGw8Params(n=2, c=32, h=10, w=70, padding=0, has_bias=False),
+         [W(groups=4, block_h=4, block_q=32, prefetch=2)],
+         [B(groups=4, block_h=7, block_q=32, prefetch=2)]),
+        (Conv2dGw8Params(n=4, c=32, h=64, w=512, padding=1, has_bias=False),
+         [W(groups=4, block_h=8, block_q=64, prefetch=4), W(groups=4, block_h=16, block_q=128, prefetch=2, two_stage=1)],
+         [B(groups=4, block_h=14, block_q=64, prefetch=4), B(groups=4, block_h=0, block_q=128, prefetch=2, block_n_iters=2, split=2)]),
+        (Conv2dGw8Params(n=2, c=64, h=20, w=1024, padding=1, has_bias=True),
+         [W(groups=8, block_h=7, block_q=128, prefetch=2), W(groups=4, block_h=20, block_q=256, prefetch=2, split=2)],
+         [B(groups=8, block_h=7, block_q=64, prefetch=2), B(groups=4, block_h=0, block_q=128, prefetch=2, split=2)]),
+    ]  # fmt: skip
+    for params, wconfigs, bconfigs in cases:
+        run_grad_kernel_test(conv2d_gw8_wgrad_kernel_factory, params, configs=wconfigs)
+        run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params, configs=bconfigs)
 
 
 # shapes the fused backward kernel has a configuration for: any padding, odd and even filter

@@ -13,6 +13,7 @@ from spio_amd.kernels import (
     Conv2dGw8Config,
     Conv2dGw8Params,
     KernelCache,
+    KernelFactory,
     KernelKey,
     KernelParamsLogger,
     LaunchParams,
@@ -72,8 +73,9 @@ def test_every_shape_has_legal_configs(igrad):
 
 def test_model_shapes_and_wide_rows_get_mfma_kernels(capsys):
     """No performance cliff onto the any-shape kernel: every model-derived shape (at its full
-    batch) and rows up to 128 pixels wide have an MFMA configuration in every family, and a
-    shape that has none (here: a row too wide for the LDS ring) says so on first use."""
+    batch) and rows of any width (column blocks: 224, 384, 512, 1024 and 4000 pixels) have an
+    MFMA configuration in every family, the fused backward kernel included for 3x3 and 5x5
+    filters; a request that has only the any-shape kernel says so on first use."""
     from helpers import GOLDEN
 
     with open(os.path.join(GOLDEN, "conv2d_gw8_model_shapes.json"), encoding="utf-8") as f:
@@ -82,16 +84,26 @@ def test_model_shapes_and_wide_rows_get_mfma_kernels(capsys):
                               r=d["r"], s=d["s"], has_bias=d["has_bias"]) for d in rows]  # fmt: skip
     shapes += [Conv2dGw8Params(n=8, c=c, h=64, w=w) for c in (64, 256) for w in (64, 96, 128)]
     shapes += [Conv2dGw8Params(n=8, c=256, h=64, w=64, r=7, s=7, padding=3)]
-    for params in shapes:
+    wide = [Conv2dGw8Params(n=2, c=c, h=20, w=w, r=r, s=r, padding=r // 2, has_bias=b)
+            for w in (224, 384, 512, 1024, 4000) for c, r, b in ((64, 3, False), (32, 5, True), (256, 3, True))]  # fmt: skip
+    wide += [Conv2dGw8Params(n=2, c=64, h=20, w=w, r=7, s=7, padding=3) for w in (224, 512, 1024)]
+    for params in shapes + wide:
         for factory, kw in ((conv2d_gw8_kernel_factory, {}), (conv2d_gw8_kernel_factory, {"igrad": True}),
                             (conv2d_gw8_wgrad_kernel_factory, {})):  # fmt: skip
             configs = factory.configs(params, ATTR, **kw)
             assert any(c.variant == "mfma" for c in configs), f"{factory.get_full_kernel_name(params, **kw)}: direct only"
+    for params in wide:
+        if params.r <= 5:
+            configs = list(conv2d_gw8_bgrad_kernel_factory.configs(params, ATTR))
+            assert configs and all(c.block_q % 32 == 0 for c in configs), f"fused backward: none for {params.encode()}"
+            if params.w >= 512:
+                assert all(c.block_q > 0 for c in configs)
 
-    # the cliff is announced where it remains
+    # the cliff is announced where a request has nothing but the any-shape kernel
     huge = Conv2dGw8Params(n=1, c=64, h=8, w=4000)
-    configs = conv2d_gw8_kernel_factory.configs(huge, ATTR)
-    assert [c.variant for c in configs] == ["direct"]
+    direct_only = KernelFactory(Conv2dGw8Params, Conv2dGw8Config, None, kernel_name="spio_conv2d_gw8_fprop",
+                                configs=lambda p, a: [Conv2dGw8Config(variant="direct")],
+                                kernel_spec=None)  # fmt: skip
 
     class Stop(Exception):
         pass
@@ -105,7 +117,7 @@ def test_model_shapes_and_wide_rows_get_mfma_kernels(capsys):
     kernel_cache.compile_and_load_kernel = no_compile
     try:
         with pytest.raises(Stop):
-            Tuner().best_kernel(conv2d_gw8_kernel_factory, huge, 0, ATTR)
+            Tuner().best_kernel(direct_only, huge, 0, ATTR)
     finally:
         kernel_cache.compile_and_load_kernel = saved
     assert "no MFMA configuration fits" in capsys.readouterr().err
