@@ -60,6 +60,9 @@ using namespace spio;
 #ifndef SPIO_BQ
 #define SPIO_BQ 0
 #endif
+#ifndef SPIO_PARTIALS
+#define SPIO_PARTIALS 0
+#endif
 #ifndef SPIO_TS
 #define SPIO_TS 1
 #endif
@@ -181,6 +184,14 @@ constexpr int RCH = (TS == 1 && WAVES * kR * NBLK * 512 <= 96 * 1024) ? kR : 1;
 constexpr int SCRATCH_FLOATS = RCH * NBLK * 128;  // per wave: row-slot halves
 constexpr int RED_FLOATS = GB * (TS - 1) * NBLK * 128;
 constexpr int GROUP_FLOATS = kR * kS * 64;
+// Two-stage publishing (SPIO_PARTIALS = 1): every workgroup stores its sums, in grad_weight order
+// (and its GB * 8 bias sums behind them), into its own block of a workspace that takes the place
+// of the grad_weight argument; the <name>_reduce kernel at the end of this file stores the sum of
+// the blocks into grad_weight (and grad_bias).  No atomics: with one-round grids all workgroups
+// reach the publish together and their atomic additions to the same lines retire one after the
+// other (14 ns each: 3.6 us for 256 workgroups at N=128, C=64, 56x56); nothing to zero first.
+constexpr int PART_FLOATS = GB * GROUP_FLOATS + (SPIO_HAS_BIAS ? GB * 8 : 0);  // one workgroup's block
+constexpr int NPART = NBLKS * PBLKS * QBLKS;  // blocks per channel block
 constexpr int PUBLISH_FLOATS =
     WAVES * SCRATCH_FLOATS + RED_FLOATS + GB * GROUP_FLOATS + (SPIO_HAS_BIAS ? WAVES * 8 : 0);
 constexpr int max3(int a, int b, int c) { return a > b ? (a > c ? a : c) : (b > c ? b : c); }
@@ -752,12 +763,24 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                 if (TS > 1) block_sync();  // the scratch is rewritten for the next filter row
             }
 }
+#if SPIO_PARTIALS
+        // this workgroup's block of the workspace: [group][k][r][s][c], then [group][k] bias sums
+        float* const pblock = grad_weight + ((long long)cb * NPART + (nbk * PBLKS + pb) * QBLKS + q0 / BQ) * PART_FLOATS;
+        if (ws == 0) {  // groups past the last one store their zeros: the block is read whole
+            float* gout = pblock + wg * GROUP_FLOATS;
+            wave_sync();  // lanes 0-31 staged the sums, all lanes read them
+#pragma unroll
+            for (int i = 0; i < kR * kS; ++i)
+                __builtin_nontemporal_store(wave_active ? gstage[64 * i + lane] : 0.f, gout + 64 * i + lane);
+        }
+#else
         if (wave_active && ws == 0) {
             float* gout = grad_weight + (long long)gglob * GROUP_FLOATS;
             wave_sync();  // lanes 0-31 staged the sums, all lanes read them
 #pragma unroll
             for (int i = 0; i < kR * kS; ++i) atomic_add_f32(gout + 64 * i + lane, gstage[64 * i + lane]);
         }
+#endif
 #if SPIO_HAS_BIAS
         {
             wave_sync();
@@ -774,6 +797,16 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                     bslots[wave * 8 + k4 + e] = wave_active ? accb[e] + scratch[e * 32 + lane] : 0.f;
             }
             block_sync();
+#if SPIO_PARTIALS
+            if (wave == 0) {
+                for (int i = lane; i < GB * 8; i += 64) {
+                    float v = 0.f;
+#pragma unroll
+                    for (int w2 = 0; w2 < TS; ++w2) v += bslots[(w2 * GB + i / 8) * 8 + (i & 7)];
+                    pblock[GB * GROUP_FLOATS + i] = v;
+                }
+            }
+#else
             if (wave == 0 && grad_bias != nullptr) {
                 for (int i = lane; i < GB * 8; i += 64) {
                     float v = 0.f;
@@ -782,7 +815,62 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                     if (cb * GB + i / 8 < kGroups) atomic_add_f32(grad_bias + 8 * cb * GB + i, v);
                 }
             }
+#endif
         }
 #endif
     }
 }
+
+#if SPIO_PARTIALS
+// Second stage: grad_weight (and grad_bias) = sum over the workgroups' blocks.  A workgroup of
+// 256 threads owns 8 float4 columns of one channel block (128 contiguous bytes of every block);
+// its 32 slices each add the blocks p = slice, slice + 32, ... with up to 8 loads in flight, the
+// slices are added through LDS and slice 0 stores the totals.  A block is laid out like the
+// channel block's part of grad_weight, so column `col` of channel block `cb` is the float4 at
+// grad_weight[cb * GB * GROUP_FLOATS + 4 * col]; the columns behind it are the bias sums.
+#define SPIO_CONCAT2(a, b) a##b
+#define SPIO_CONCAT(a, b) SPIO_CONCAT2(a, b)
+extern "C" __global__ void SPIO_LAUNCH_BOUNDS(256)
+SPIO_CONCAT(SPIO_KERNEL_NAME, _reduce)(float* __restrict__ grad_weight, const spio_float4* __restrict__ partials,
+                                       float* __restrict__ grad_bias) {
+    constexpr int BLOCK_F4 = PART_FLOATS / 4;  // float4 columns of one block
+    constexpr int COLS = 8;
+    constexpr int SLICES = 256 / COLS;
+    constexpr int UN = 8;
+    constexpr int WGS_PER_CB = (BLOCK_F4 + COLS - 1) / COLS;
+    __shared__ spio_float4 red[SLICES][COLS];
+    const int tid = thread_id();
+    const int cl = tid % COLS;
+    const int slice = tid / COLS;
+    const int cb = block_id() / WGS_PER_CB;
+    const int col = (block_id() % WGS_PER_CB) * COLS + cl;
+    const bool live = col < BLOCK_F4;
+    const spio_float4* base = partials + (long long)cb * NPART * BLOCK_F4 + (live ? col : 0);
+    spio_float4 sum = spio_float4{0.f, 0.f, 0.f, 0.f};
+    for (int p0 = slice; p0 < NPART; p0 += SLICES * UN) {
+        spio_float4 v[UN];
+#pragma unroll
+        for (int i = 0; i < UN; ++i) {
+            const int p = p0 + i * SLICES;
+            v[i] = spio_float4{0.f, 0.f, 0.f, 0.f};
+            if (p < NPART) v[i] = __builtin_nontemporal_load(base + (long long)p * BLOCK_F4);
+        }
+#pragma unroll
+        for (int i = 0; i < UN; ++i) sum += v[i];
+    }
+    red[slice][cl] = sum;
+    block_sync();
+    if (slice == 0 && live) {
+#pragma unroll 4
+        for (int i = 1; i < SLICES; ++i) sum += red[i][cl];
+        const int f = 4 * col;  // float index inside the block
+        if (f < GB * GROUP_FLOATS) {
+            if (cb * GB + f / GROUP_FLOATS < kGroups)
+                *reinterpret_cast<spio_float4*>(grad_weight + (long long)cb * GB * GROUP_FLOATS + f) = sum;
+        } else if (grad_bias != nullptr) {
+            const int k = cb * GB * 8 + (f - GB * GROUP_FLOATS);
+            if (k < kC) *reinterpret_cast<spio_float4*>(grad_bias + k) = sum;
+        }
+    }
+}
+#endif

@@ -31,8 +31,8 @@
 //     added with instructions that cover 64 consecutive floats (two full
 //     lines): the fewest line operations possible.  SPIO_PARTIALS=1 stores each
 //     workgroup's sums into its own partial image of a workspace with plain
-//     stores, and the small <name>_reduce kernel below folds the partial images
-//     into grad_weight.  (Reducing inside the kernel by "the last workgroup of
+//     stores, and the small <name>_reduce kernel below stores the sum of the
+//     partial images into grad_weight (which then needs no zero fill).  (Reducing inside the kernel by "the last workgroup of
 //     a group to finish" was measured and rejected: the device-scope
 //     release/acquire fences it needs write back and invalidate the L2 of an
 //     XCD and cost more than the atomics they save.)
@@ -629,7 +629,8 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
 }
 
 #if SPIO_PARTIALS
-// Second stage: grad_weight += sum over the partial blocks.  A workgroup owns 32 float4 columns
+// Second stage: grad_weight = sum over the partial blocks (stored whole: a caller that runs the
+// two-stage kernel need not zero grad_weight first).  A workgroup owns 32 float4 columns
 // of one channel block (512 contiguous bytes of every partial block: half a wave per load
 // instruction); its 8 slices each add the blocks p = slice, slice + 8, ... with 4 loads in
 // flight, the slices are added through LDS and slice 0 adds the total onto grad_weight.  (With 8
@@ -683,7 +684,7 @@ SPIO_CONCAT(SPIO_KERNEL_NAME, _reduce)(float* __restrict__ grad_weight, const sp
         if (cb * GB + g < kGroups && s < kS) {
             spio_float4* dst =
                 reinterpret_cast<spio_float4*>(grad_weight + (((long long)k * kR + r) * kS + s) * 8 + (l32 & 7));
-            *dst = *dst + sum;
+            *dst = sum;
         }
     }
 }

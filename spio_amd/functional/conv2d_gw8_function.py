@@ -198,19 +198,24 @@ def conv2d_gw8_backward_op(
     grad_input = None
     fused = fused_backward_kernel(params, inputs.device) if needs_input_grad and needs_weight_grad else None
     if fused is not None:
-        # one pass over grad_output for both gradients (and grad_bias when the layer has a bias)
-        grad_weight = torch.zeros_like(weight, dtype=torch.float32)
+        # one pass over grad_output for both gradients (and grad_bias when the layer has a bias);
+        # atomic kernels add into zeroed tensors, two-stage ones store them whole
+        make = torch.empty_like if fused.kernel_spec.overwrites_output else torch.zeros_like
+        grad_weight = make(weight, dtype=torch.float32)
         grad_input = torch.empty_like(inputs)
         if params.has_bias:
             if needs_bias_grad:
-                grad_bias = torch.zeros(params.c, dtype=torch.float32, device=inputs.device)
+                alloc = torch.empty if fused.kernel_spec.overwrites_output else torch.zeros
+                grad_bias = alloc(params.c, dtype=torch.float32, device=inputs.device)
             fused(grad_input, grad_weight, inputs, grad_output, weight, grad_bias)
         else:
             fused(grad_input, grad_weight, inputs, grad_output, weight)
     elif needs_weight_grad:
-        # The kernel accumulates into grad_weight, so it starts from zero; fp32.
-        grad_weight = torch.zeros_like(weight, dtype=torch.float32)
+        # An atomic kernel accumulates into grad_weight, so it starts from zero; a two-stage one
+        # stores it whole; fp32.
         kernel = conv2d_gw8_wgrad_kernel_factory.get_kernel(params, inputs.device)
+        make = torch.empty_like if kernel.kernel_spec.overwrites_output else torch.zeros_like
+        grad_weight = make(weight, dtype=torch.float32)
         if params.has_bias:
             # With a bias the weight-gradient kernel also sums grad_output per channel while it
             # streams it (the reference runs a separate reduction, conv2d_gw8_function.py:134-136).

@@ -9,7 +9,8 @@ every other padding is one on a larger domain in which the input and the output
 sit at fitting offsets (`bgrad_domain`).
 
 Kernel arguments: (grad_input, grad_weight, x, grad_output, weight[, grad_bias]);
-grad_weight (and grad_bias) are accumulated into, so the caller zeroes them first.
+grad_weight (and grad_bias) are accumulated into, so the caller zeroes them first, unless the
+configuration is two-stage (`KernelSpec.overwrites_output`): then both are stored whole.
 """
 
 from dataclasses import dataclass, replace
@@ -53,6 +54,11 @@ class Conv2dGw8BgradConfig:
             cache policy (the second reader can hit in L2), the others with the non-temporal hint.
         xcd_chunk: consecutive tiles that go to the same XCD before the next run goes to the next
             one; 0 = one contiguous range of tiles per XCD.
+        two_stage: 1 = workgroups store their grad_weight (and grad_bias) sums into blocks of a
+            workspace and a second kernel stores the blocks' sum into grad_weight and grad_bias,
+            which then need no zero fill; 0 = workgroups add into zeroed tensors with fp32
+            atomics.  Atomic additions of different workgroups to one line retire one after the
+            other, and in a one-round grid all workgroups publish at the same time.
         block_q: columns per workgroup (0: the whole width; else a multiple of 32 with
             block_n = 1).  The workgroup stages block_q + S - 1 columns of x and of grad_output, so
             rows of any width fit.
@@ -67,6 +73,7 @@ class Conv2dGw8BgradConfig:
     halo_cached: int = 1
     xcd_chunk: int = 4
     block_q: int = 0
+    two_stage: int = 0
 
 
 def bgrad_is_supported(params: Conv2dGw8Params) -> bool:
@@ -231,6 +238,9 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None) -> List[Conv2dGw8Bgr
     configs += [replace(cfg, prefetch=8) for cfg in first[:3] if _config_is_legal(params, replace(cfg, prefetch=8))]
     # ... and the other memory-system policies
     configs += [replace(cfg, halo_cached=hc, xcd_chunk=ch) for cfg in first[:2] for hc, ch in ((0, 4), (1, 0))]
+    # ... and two-stage publishing for the leaders of every height
+    configs += [replace(cfg, two_stage=1) for cfg in list(configs) if cfg.prefetch == 4 and cfg.halo_cached == 1
+                and cfg.xcd_chunk == 4][:2 * GEOMETRIES_PER_HEIGHT]  # fmt: skip
     return configs
 
 
@@ -246,7 +256,19 @@ def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8BgradConfig, _dev
                    SPIO_HAS_BIAS=int(params.has_bias))  # fmt: skip
     if config.block_q:
         defines["SPIO_BQ"] = config.block_q
-    return KernelSpec(defines, LaunchParams(grid=g["NUM_BLOCKS"], block=g["THREADS"]), SOURCE, notes=g)
+    spec = KernelSpec(defines, LaunchParams(grid=g["NUM_BLOCKS"], block=g["THREADS"]), SOURCE, notes=g)
+    if config.two_stage:
+        # one block per workgroup: its groups' grad_weight values, then its 8 bias sums per group
+        part_floats = config.groups * params.r * params.s * 64 + (config.groups * 8 if params.has_bias else 0)
+        npart = g["NBLKS"] * g["PBLKS"] * g["QBLKS"]
+        defines.update(SPIO_PARTIALS=1)
+        spec.workspace_bytes = g["GBLKS"] * npart * part_floats * 4
+        spec.workspace_arg = 1  # the workspace takes the place of grad_weight
+        spec.epilogue_suffix = "_reduce"
+        spec.epilogue_extra_args = (5,)  # grad_bias, or None where there is none
+        spec.epilogue_launch_params = LaunchParams(grid=g["GBLKS"] * divup(part_floats // 4, 8), block=256)
+        spec.overwrites_output = True
+    return spec
 
 
 def _make_test_args(params: Conv2dGw8Params, device):

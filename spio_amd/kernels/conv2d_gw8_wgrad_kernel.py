@@ -51,7 +51,8 @@ class Conv2dGw8WgradConfig:
         split: waves sharing the 32-pixel chunks of one group; their sums are added in LDS
             before publishing, so bigger workgroups do not publish more.
         two_stage: 1 = workgroups store partial sums to a workspace and a second kernel
-            reduces them; 0 = workgroups add into grad_weight with fp32 atomics.
+            stores their sum into grad_weight (no zero fill needed, deterministic); 0 =
+            workgroups add into a zeroed grad_weight with fp32 atomics.
         variant: "mfma" (row-streaming MFMA kernel) or "direct" (any shape).
         block_q: grad_output columns per workgroup (0: the whole width); the workgroup stages
             block_q + S - 1 columns of x opposite them, so rows of any width fit.
@@ -233,6 +234,7 @@ def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig, _dev
         defines.update(SPIO_PARTIALS=1)
         spec.workspace_bytes = num_partials * cols * 16
         spec.epilogue_suffix = "_reduce"
+        spec.overwrites_output = True  # the second stage stores grad_weight whole
         # one workgroup per 32 float4 columns (cols is a multiple of 32 per channel block)
         spec.epilogue_launch_params = LaunchParams(grid=cols // 32, block=256)
     return spec

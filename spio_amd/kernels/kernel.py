@@ -34,11 +34,16 @@ class KernelSpec:
     max_dynamic_lds: Optional[int] = None
     notes: Dict[str, object] = field(default_factory=dict)
     # Two-stage kernels: the main kernel receives a workspace of `workspace_bytes` in place of
-    # its first argument, then `<kernel name><epilogue_suffix>` runs with (first argument,
-    # workspace) under `epilogue_launch_params`.
+    # argument `workspace_arg`, then `<kernel name><epilogue_suffix>` runs with (that argument,
+    # workspace, and the arguments listed in `epilogue_extra_args`) under `epilogue_launch_params`.
     workspace_bytes: int = 0
     epilogue_suffix: Optional[str] = None
     epilogue_launch_params: Optional[LaunchParams] = None
+    workspace_arg: int = 0
+    epilogue_extra_args: tuple = ()
+    # True: the kernel (its last stage) stores the tensor at `workspace_arg` whole, so the caller
+    # need not zero it; False: the kernel adds into it
+    overwrites_output: bool = False
 
 
 
@@ -175,19 +180,32 @@ class Kernel:
             elif static_workspace:
                 ep = spec.epilogue_launch_params
                 nbytes = spec.workspace_bytes
-                self.function.launch_scratch(lp.grid, lp.block, (None,) + args[1:], 0, nbytes,
+                wa = spec.workspace_arg
+                self.function.launch_scratch(lp.grid, lp.block, self._stage_args(args, None)[0], wa, nbytes,
                                              lp.shared_mem_bytes, stream)  # fmt: skip
-                self.epilogue_function.launch_scratch(ep.grid, ep.block, (args[0], None), 1, nbytes,
+                self.epilogue_function.launch_scratch(ep.grid, ep.block, self._stage_args(args, None)[1], 1, nbytes,
                                                       ep.shared_mem_bytes, stream)  # fmt: skip
             else:
                 workspace = self._workspace(device)
-                self.function.launch(lp.grid, lp.block, (workspace,) + args[1:], lp.shared_mem_bytes, stream)
+                main_args, epilogue_args = self._stage_args(args, workspace)
+                self.function.launch(lp.grid, lp.block, main_args, lp.shared_mem_bytes, stream)
                 ep = spec.epilogue_launch_params
-                self.epilogue_function.launch(ep.grid, ep.block, (args[0], workspace), ep.shared_mem_bytes, stream)
+                self.epilogue_function.launch(ep.grid, ep.block, epilogue_args, ep.shared_mem_bytes, stream)
             if timer is not None:
                 stop.record()
         except Exception as e:
             raise ValueError(f"Error in kernel {self}") from e
+
+    def _stage_args(self, args, workspace):
+        """Arguments of the two stages of a two-stage kernel: the main stage gets the workspace in
+        place of argument `workspace_arg`, the second stage that argument, the workspace and the
+        listed extra arguments (missing trailing ones, e.g. an absent grad_bias, become None)."""
+        spec = self.kernel_spec
+        wa = spec.workspace_arg
+        args = tuple(args)
+        main = args[:wa] + (workspace,) + args[wa + 1:]
+        extra = tuple(args[i] if i < len(args) else None for i in spec.epilogue_extra_args)
+        return main, (args[wa], workspace) + extra
 
     def _workspace(self, device) -> torch.Tensor:
         """Scratch for the partial results of a two-stage kernel (from torch's caching allocator)."""
@@ -211,9 +229,10 @@ class Kernel:
         sets = []
         for kargs in prepared:
             ws = self._workspace(device)
+            main_args, epilogue_args = self._stage_args(kargs, ws)
             sets.append([
-                (self.function, lp.grid, lp.block, lp.shared_mem_bytes, [ws] + kargs[1:]),
-                (self.epilogue_function, ep.grid, ep.block, ep.shared_mem_bytes, [kargs[0], ws]),
+                (self.function, lp.grid, lp.block, lp.shared_mem_bytes, list(main_args)),
+                (self.epilogue_function, ep.grid, ep.block, ep.shared_mem_bytes, list(epilogue_args)),
             ])  # fmt: skip
         return launch_sequence_timed(sets, stream, warmup, iters)
 

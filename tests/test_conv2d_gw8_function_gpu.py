@@ -155,21 +155,61 @@ def test_fused_backward_choice(monkeypatch):
     assert fused_backward_kernel(same, dev) is None
 
 
-def test_wgrad_accumulates_into_its_output():
-    """The weight-gradient kernel adds to grad_weight: two launches give exactly twice one
-    launch's contribution (up to the order of fp32 atomics)."""
-    from spio_amd.kernels import conv2d_gw8_wgrad_kernel_factory
+def test_atomic_kernels_accumulate_and_two_stage_kernels_overwrite():
+    """A weight-gradient (or fused backward) kernel that publishes with atomics adds to
+    grad_weight: two launches give twice one launch's contribution (up to the order of fp32
+    atomics).  A two-stage kernel stores grad_weight (and grad_bias) whole: whatever they held
+    before is gone, which is why the operator does not zero them for such a kernel."""
+    from spio_amd.hip import get_device_attributes
+    from spio_amd.kernels import (
+        Conv2dGw8BgradConfig,
+        Conv2dGw8WgradConfig,
+        conv2d_gw8_bgrad_kernel_factory,
+        conv2d_gw8_wgrad_kernel_factory,
+    )
 
-    p = Conv2dGw8Params(n=2, c=16, h=8, w=8)
-    x, w, _b, dy = oracle.make_args(p.n, p.c, p.h, p.w, 3, 3, 1, 1, False, 0)
-    kernel = conv2d_gw8_wgrad_kernel_factory.get_kernel(p, torch.device("cuda", 0))
-    dw = torch.zeros(p.weight_shape, device="cuda").contiguous(memory_format=torch.channels_last)
-    kernel(dw, to_gpu(x), to_gpu(dy))
-    once = dw.clone()
-    kernel(dw, to_gpu(x), to_gpu(dy))
-    torch.cuda.synchronize()
-    assert torch.allclose(dw, 2 * once, rtol=1e-5, atol=1e-4)
-    oracle.check_close(once, oracle.grads_torch(x, w, None, dy, 1, 1)[1], acc_depth=128, what="wgrad once")
+    attr = get_device_attributes(0)
+    p = Conv2dGw8Params(n=6, c=16, h=8, w=8, has_bias=True)
+    x, w, b, dy = oracle.make_args(p.n, p.c, p.h, p.w, 3, 3, 1, 1, True, 0)
+    _dx_e, dw_e, db_e = oracle.grads_torch(x, w, b, dy, 1, 1)
+    xg, wg, dyg = to_gpu(x), to_gpu(w), to_gpu(dy)
+
+    def fresh(value):
+        dw = torch.full(p.weight_shape, value, device="cuda").contiguous(memory_format=torch.channels_last)
+        return dw, torch.full((p.c,), value, device="cuda")
+
+    for two_stage in (0, 1):
+        wk = conv2d_gw8_wgrad_kernel_factory.make_kernel(
+            p, Conv2dGw8WgradConfig(groups=2, block_h=4, block_n=2, prefetch=2, two_stage=two_stage), attr)
+        bk = conv2d_gw8_bgrad_kernel_factory.make_kernel(
+            p, Conv2dGw8BgradConfig(groups=2, block_h=4, block_n=2, prefetch=2, two_stage=two_stage), attr)
+        for kernel, call in ((wk, lambda dw, db: wk(dw, xg, dyg, db)),
+                             (bk, lambda dw, db: bk(torch.empty_like(xg), dw, xg, dyg, wg, db))):  # fmt: skip
+            kernel.compile()
+            kernel.load(0)
+            assert kernel.kernel_spec.overwrites_output == bool(two_stage)
+            dw, db = fresh(0.0)
+            call(dw, db)
+            once_w, once_b = dw.clone(), db.clone()
+            oracle.check_close(once_w, dw_e, acc_depth=p.n * 64, what=f"{kernel.kernel_name} once")
+            oracle.check_close(once_b, db_e, acc_depth=p.n * 64, what=f"{kernel.kernel_name} bias once")
+            call(dw, db)
+            torch.cuda.synchronize()
+            factor = 1 if two_stage else 2
+            assert torch.allclose(dw, factor * once_w, rtol=1e-5, atol=1e-4)
+            # grad_bias: the fused kernel's second stage stores it; the weight-gradient kernel's
+            # two-stage mode still adds it with atomics
+            bias_factor = 1 if (two_stage and kernel is bk) else 2
+            assert torch.allclose(db, bias_factor * once_b, rtol=1e-5, atol=1e-3)
+            if two_stage:  # garbage in the outputs does not matter
+                dw, db = fresh(123.0)
+                if kernel is wk:
+                    db.zero_()
+                call(dw, db)
+                torch.cuda.synchronize()
+                assert torch.allclose(dw, once_w, rtol=1e-5, atol=1e-4)
+                assert torch.allclose(db, once_b, rtol=1e-5, atol=1e-3)
+            kernel.unload()
 
 
 def test_non_channels_last_arguments_are_accepted():

@@ -160,6 +160,29 @@ def test_bgrad_sanity(params):
     run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params)
 
 
+def test_bgrad_two_stage():
+    """Fused backward kernel with two-stage publishing: blocks of partial sums and the second
+    kernel that stores their sum.  Channel blocks with missing groups, row and column blocks,
+    images side by side, image blocks per workgroup, split groups, with and without a bias."""
+    C = Conv2dGw8BgradConfig
+    cases = [
+        (Conv2dGw8Params(n=5, c=24, h=20, w=28, padding=1, has_bias=True),
+         [C(groups=2, block_h=7, block_n=2, block_n_iters=1, prefetch=2, two_stage=1),
+          C(groups=3, block_h=0, block_n=2, block_n_iters=2, prefetch=4, split=2, two_stage=1)]),
+        (Conv2dGw8Params(n=3, c=72, h=19, w=40, padding=1, has_bias=False),
+         [C(groups=4, block_h=7, block_n=1, block_n_iters=1, prefetch=2, two_stage=1),
+          C(groups=9, block_h=14, block_n=1, block_n_iters=2, prefetch=2, two_stage=1)]),
+        (Conv2dGw8Params(n=2, c=40, h=9, w=9, r=5, s=5, padding=2, has_bias=True),
+         [C(groups=5, block_h=0, block_n=2, prefetch=2, two_stage=1)]),
+        (Conv2dGw8Params(n=3, c=24, h=9, w=150, padding=1, has_bias=True),
+         [C(groups=3, block_h=4, block_q=64, prefetch=2, two_stage=1)]),
+        (Conv2dGw8Params(n=5, c=32, h=17, w=21, r=4, s=4, padding=(0, 3), has_bias=True),
+         [C(groups=4, block_h=5, block_n=1, block_n_iters=1, prefetch=2, two_stage=1)]),
+    ]  # fmt: skip
+    for params, configs in cases:
+        run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params, configs=configs)
+
+
 def test_bgrad_when_the_image_size_changes():
     """Paddings other than (R-1)/2, and even filter sizes: the kernel works on a domain that holds
     both tensors at offsets that reproduce the padding.  Row blocks that lie partly or wholly
