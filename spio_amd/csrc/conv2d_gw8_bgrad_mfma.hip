@@ -510,6 +510,7 @@ SPIO_KERNEL_NAME(spio_uint4* __restrict__ grad_input, float* __restrict__ grad_w
                 v.u = *reinterpret_cast<const spio_uint4*>(ostage + obuf * OUT_ROW_BYTES + o_lds[l]);
                 __builtin_amdgcn_raw_buffer_store_b128(v.i, rs, (int)(o_voff[l] + row_off), 0, AUX_NT);
             }
+            store_group_end();
         };
 
         for (int tb = 0; tb < ROWS; tb += UNROLL) {

@@ -458,6 +458,7 @@ SPIO_DEVICE void conv_rows(spio_uint4* __restrict__ dst, const spio_uint4* __res
             v.u = *(lds_u4p)(ostage + obuf * OUT_ROW_BYTES + out_lds[s]);
             __builtin_amdgcn_raw_buffer_store_b128(v.i, rs, (int)(out_voff[s] + row_off), 0, AUX_ST);
         }
+        store_group_end();
     };
 
     // Rows above and below the image are rows of zeros in the ring; their products are skipped (a

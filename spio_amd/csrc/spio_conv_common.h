@@ -94,6 +94,23 @@ SPIO_DEVICE void store_stream(spio_uint4 v, spio_uint4* p) {
 #endif
 }
 
+// Closes a group of 16-byte buffer stores.  Such a store reads its data registers for a few
+// cycles after it issues; an instruction that writes one of them in the very next slot can have
+// its value stored instead (seen on gfx950 as stray values in the first two channels of some
+// pixels).  The compiler keeps that slot free only for some operand forms of the store, so the
+// kernels do not rely on it: nothing is scheduled across this point, and the wait state between
+// the last store and whatever follows is explicit.
+#ifndef SPIO_STORE_GUARD
+#define SPIO_STORE_GUARD 1
+#endif
+SPIO_DEVICE void store_group_end() {
+#if SPIO_STORE_GUARD
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_nop 0");
+    __builtin_amdgcn_sched_barrier(0);
+#endif
+}
+
 // Device-scope fp32 add without a return value.
 SPIO_DEVICE void atomic_add_f32(float* address, float value) {
     __hip_atomic_fetch_add(address, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

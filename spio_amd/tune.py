@@ -56,8 +56,11 @@ def tune_model(model, inputs: Sequence, backward: bool = True, max_configs: Opti
          (`KernelCache.update_overlay`) and runs the model `warmup + iters` times over `inputs`
          (a list of input batches, rotated) while `LaunchTimer` times each launch with HIP events:
          kernels are timed with the cache state and neighbours they have in the model;
-      4. a round whose model output disagrees with the first round's is discarded as a whole
-         (one of its configurations computes something else);
+      4. every round's model output and, with `backward`, the gradients of the model's
+         parameters after its first iteration are kept; the rounds are then compared with each
+         other and those that disagree with the largest group of agreeing rounds are discarded
+         as a whole (one of their configurations computes something else, in the forward or in
+         the backward pass; a wrong first round is outvoted like any other);
       5. the fastest candidate of every kernel is written to the tuning records (the user
          record file, or `record_path`), the caches are cleared, and the next request for each
          of these kernels compiles the recorded winner.
@@ -115,7 +118,8 @@ def tune_model(model, inputs: Sequence, backward: bool = True, max_configs: Opti
     # fused data+weight gradient kernel or the two separate ones, every round is run both ways so
     # that all three families get their in-situ times.
     times: Dict[Any, Dict[int, float]] = {kp: {} for kp in unique}
-    reference_out = None
+    round_times = []  # (idx, mode, {kp: us}) per round
+    round_results = []  # what the model computed in that round: [output, gradients...]
     discarded = []
     has_fused = any(kp.kernel_factory.get_kernel_name(**dict(kp.kernel_kwargs)).endswith("bgrad") for kp in unique)
     saved_mode = os.environ.get("SPIO_FUSED_BACKWARD")
@@ -132,11 +136,15 @@ def tune_model(model, inputs: Sequence, backward: bool = True, max_configs: Opti
             caches[cid].update_overlay(overlay)
         reset_fused_backward_choices()
         try:
+            if backward:
+                model.zero_grad(set_to_none=True)
             with LaunchTimer() as timer:
                 for i in range(warmup + iters):
                     out = run(inputs[i % len(inputs)])
                     if i == 0:
-                        first_out = out.float().clone()
+                        computed = [out.float().clone()]
+                        if backward:
+                            computed += [p.grad.float().clone() for p in model.parameters() if p.grad is not None]
                 averages = timer.averages(skip=warmup)
         finally:
             for cache in caches.values():
@@ -148,14 +156,26 @@ def tune_model(model, inputs: Sequence, backward: bool = True, max_configs: Opti
                     os.environ.pop("SPIO_FUSED_BACKWARD", None)
                 else:
                     os.environ["SPIO_FUSED_BACKWARD"] = saved_mode
-        if reference_out is None:
-            reference_out = first_out
-        elif not torch.allclose(first_out, reference_out, rtol=2e-2, atol=2e-2 * float(reference_out.abs().max())):
+        round_results.append(computed)
+        round_times.append((idx, mode, {kp: averages[kernel] for kp, kernel in choice.items()
+                                        if idx < len(table[kp]) and kernel in averages}))  # fmt: skip
+
+    def agree(a, b):
+        return len(a) == len(b) and all(
+            x.shape == y.shape and torch.allclose(x, y, rtol=2e-2, atol=2e-2 * max(float(y.abs().max()), 1e-6))
+            for x, y in zip(a, b)
+        )
+
+    # the reference is the round most other rounds agree with
+    votes = [sum(agree(a, b) for b in round_results) for a in round_results]
+    reference = round_results[votes.index(max(votes))]
+    for (idx, mode, per_kernel), computed in zip(round_times, round_results):
+        if not agree(computed, reference):
             discarded.append((idx, mode))
             continue
-        for kp, kernel in choice.items():
-            if idx < len(table[kp]) and kernel in averages:
-                times[kp][idx] = averages[kernel]
+        for kp, us in per_kernel.items():
+            times[kp][idx] = us
+    del round_results, reference
 
     # 5. record the winners
     results = []
@@ -181,7 +201,7 @@ def tune_model(model, inputs: Sequence, backward: bool = True, max_configs: Opti
         cache.clear_cache()
     reset_fused_backward_choices()
     if discarded:
-        print(f"spio: tune_model discarded rounds {discarded}: model output differed from the first round")
+        print(f"spio: tune_model discarded rounds {discarded}: output or gradients differed from the other rounds")
     return results
 
 
