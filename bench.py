@@ -188,6 +188,8 @@ def kernel_entry(kernel, arg_sets, nbytes, iters, min_seconds=MIN_TIMED_SECONDS)
         "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
         "config": dict(vars(kernel.config)),
         "kernel": kernel.kernel_name,
+        "source": kernel.kernel_source_file,
+        "source_digest": source_digest(kernel.kernel_source_file),
     }
 
 

@@ -6,7 +6,11 @@ csrc/spio_hip_scratch.hip and csrc/spio_hip_fill.hip (hipcc, gfx950: the static
 device workspace with the launch that uses it, and the zero-fill kernel; they
 link the HIP runtime by its soname, so the copy a host framework has already
 mapped is the one used).  hipcc cross-compiles, so this builds on machines
-without a GPU.
+without a GPU.  Loading is another matter: because of the device translation
+units the library has libamdhip64 as a link-time dependency and registers its
+code objects when it is dlopen'ed, so every process that loads it, the
+host-only tests and tools included, needs the HIP runtime library installed
+(a GPU is not needed to load it).
 
 `check_kernels()` compiles every HIP kernel source for gfx950 with hipcc for
 a list of representative shape specialisations; at run time the same sources

@@ -24,5 +24,11 @@ class KernelParams:
 
     @property
     def key(self) -> KernelKey:
+        """The key KernelCache.get files this request under: a device without an index means the
+        current device, as it does there."""
         idx = self.device.index
-        return KernelKey(device_ordinal=0 if idx is None else idx, params=self.params)
+        if idx is None:
+            import torch  # pylint: disable=import-outside-toplevel
+
+            idx = torch.cuda.current_device()
+        return KernelKey(device_ordinal=idx, params=self.params)
