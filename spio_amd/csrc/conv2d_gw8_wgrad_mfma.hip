@@ -69,6 +69,9 @@ using namespace spio;
 #ifndef SPIO_HAS_BIAS
 #define SPIO_HAS_BIAS 0
 #endif
+#ifndef SPIO_PIPE
+#define SPIO_PIPE 0
+#endif
 
 namespace {
 
@@ -90,14 +93,34 @@ constexpr int ND = kR + 1;     // values of delta
 // fixed block of 8 columns, spio/kernels/conv2d_gw8_wgrad_kernel.py:40).  0 = the whole width.
 constexpr int BQ = SPIO_BQ > 0 ? SPIO_BQ : kQ;
 constexpr int QBLKS = (kQ + BQ - 1) / BQ;
-constexpr int WPI = BQ + kS - 1;  // padded width of one image (block): W + 2*px for whole rows
+constexpr int WPI = BQ + kS - 1;  // x cells staged per image (block): W + 2*px for whole rows
 constexpr int F = NB * WPI;
-constexpr int KSPAN = (NB - 1) * WPI + BQ;  // flattened pixels that carry dy
-constexpr int KC = (KSPAN + 31) / 32;       // 32-pixel chunks
-constexpr int FPX = 32 * KC + S2 - 1;
+// Where the images of a staged row sit.  dy pixel q of image i lies at flattened pixel
+// off(i) + q and meets, for column tap s, the x pixel at off(i) + q + s; x column c of image i
+// lies at off(i) + c + px.  Between the data of two images GAP = max(px, S-1-px) zero cells are
+// enough: the right halo of one image is the left halo of the next.  The contraction runs over
+// 32-pixel chunks of the dy row; where a chunk holds IPC >= 1 whole images and that takes fewer
+// chunks than the images laid end to end, every chunk gets its own IPC images (14x14 images
+// under a 7x7 filter: two per chunk, 28 of 32 pixels, instead of four in three chunks), and the
+// x row, whose pixels q + s reach S-1 cells past a chunk, is staged as chunks XCP cells apart.
+#ifndef SPIO_SHARED_HALO
+#define SPIO_SHARED_HALO 1
+#endif
+constexpr int GAP = kPadX > kS - 1 - kPadX ? kPadX : kS - 1 - kPadX;
+constexpr int IP = (SPIO_BQ > 0 || !SPIO_SHARED_HALO) ? WPI : BQ + GAP;  // pitch of the images in a run
+constexpr int IPC_MAX = (32 + IP - BQ) / IP;                             // whole images per 32-pixel chunk
+constexpr int KC_FLAT = ((NB - 1) * IP + BQ + 31) / 32;
+constexpr int KC_PACKED = IPC_MAX > 0 ? (NB + IPC_MAX - 1) / IPC_MAX : KC_FLAT;
+constexpr bool kPacked = SPIO_SHARED_HALO && KC_PACKED < KC_FLAT;
+constexpr int IPC = kPacked ? IPC_MAX : NB;  // images per run: a chunk, or the whole row
+constexpr int KC = kPacked ? KC_PACKED : KC_FLAT;  // 32-pixel chunks
+constexpr int XCP = kPacked ? 16 * ((32 + S2 - 1 + 15) / 16) : 32;  // x cells from chunk to chunk
+constexpr int FPX = kPacked ? KC * XCP : 32 * KC + S2 - 1;         // x pixels the reads can touch
 constexpr int GSX = FPX + ((9 - FPX % 16) + 16) % 16;  // x group stride (pixels), = 9 mod 16
 constexpr int FPD = 32 * KC;
 constexpr int GSD = FPD + ((9 - FPD % 16) + 16) % 16;  // dy group stride
+constexpr int d_image_offset(int img) { return (img / IPC) * 32 + (img % IPC) * IP; }
+constexpr int x_image_offset(int img) { return (img / IPC) * XCP + (img % IPC) * IP; }
 constexpr int NRX = 2 * RB;                             // x ring rows: the step's rows and the next step's
 // dy ring rows: the aligned row pairs a step multiplies (R+1 rows with one row per step, up to
 // R+2 with two) plus the rows the step writes for the next one; even.  The bias sum reads the
@@ -121,6 +144,25 @@ constexpr bool kDbias = SPIO_HAS_BIAS != 0;  // also sum grad_output per channel
 // first row was staged, so a one-row filter needs one more step when the sum is wanted.
 constexpr int ROWS = BH + (kDbias && kR == 1 ? 2 : kR) - 1;
 constexpr int STEPS = (ROWS + RB - 1) / RB;  // barrier-separated steps of RB rows
+// A workgroup that owns whole images (one row block) knows at compile time which of its x rows
+// lie in the padding: the steps before the first real row would only stage dy rows, the steps
+// after the last one nothing at all.  It starts at the first step with a real x row, with the dy
+// rows up to that step staged in the prologue, and stops after the last.  (Not with the bias
+// sum, which takes its row pairs at fixed steps.)
+constexpr bool kSkipPadding = PBLKS == 1 && !kDbias;
+constexpr int T_FIRST = kSkipPadding ? kPadY : 0;
+constexpr int T_END = kSkipPadding && kH + kPadY < ROWS ? kH + kPadY : ROWS;
+constexpr int S0 = T_FIRST / RB;               // first step
+constexpr int S1 = (T_END + RB - 1) / RB;      // one past the last step
+constexpr int LEAD = S0 * RB;                  // dy rows staged ahead of the first step's own
+// A workgroup that owns whole images unrolls its step loop completely, up to SPIO_MAX_UNROLL
+// steps (every condition on the step is then known at compile time); other loops run in chunks
+// of PF steps.
+#ifndef SPIO_MAX_UNROLL
+#define SPIO_MAX_UNROLL 64
+#endif
+constexpr bool kFullUnroll = PBLKS == 1 && S1 - S0 <= SPIO_MAX_UNROLL;
+constexpr int UNROLL = kFullUnroll ? (S1 - S0 + PF - 1) / PF * PF : PF;
 constexpr int NPAIR = kR / 2 + 1;            // aligned dy row pairs one step can touch
 constexpr int CPW = (KC + TS - 1) / TS;      // 32-pixel chunks per wave
 
@@ -144,6 +186,7 @@ static_assert(LDS_UNITS * 16 <= 160 * 1024, "LDS overflow");
 static_assert(NRD % 2 == 0 && NRD >= kR + 1, "dy ring too small");
 static_assert(PF >= 2 && PF % 2 == 0, "prefetch distance must be even");
 static_assert(RB == 1 || RB == 2, "one or two rows per step");
+static_assert(LEAD + RB <= NRD, "the dy rows of the prologue fit the ring");
 constexpr int PART_WAVE_FLOATS = kR * NBLK * 4 * 32;  // floats one wave publishes (partial-block layout)
 
 
@@ -184,7 +227,7 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
     if (NUM_BLOCKS % 8 == 0) b = (b & 7) * (NUM_BLOCKS / 8) + (b >> 3);
     const int qb = b % QBLKS;  // column blocks fastest: neighbours share S - 1 columns of x
     const int q0 = qb * BQ;
-    const int pb = (b / QBLKS) % PBLKS;
+    const int pb = PBLKS == 1 ? 0 : (b / QBLKS) % PBLKS;
     const int cb = (b / (QBLKS * PBLKS)) % GBLKS;
     const int nbk = b / (QBLKS * PBLKS * GBLKS);
     const int p0 = pb * BH;
@@ -225,7 +268,9 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
         // compiler counts outstanding loads exactly and a step waits only for the rows it
         // needs (a load under a branch makes it wait for all of them, which would serialise the
         // prefetch).  Cells without data (halo columns, missing images or groups) and rows
-        // outside the tensor load a valid address and become zero when written to LDS.
+        // outside the tensor load a valid address and become zero when written to LDS.  (Threads
+        // beyond the last cell skip their LDS writes; letting them write spare cells instead, to
+        // make the writes branch-free, costs 14 % at N=256, C=256, 14x14, 7x7.)
         int x_off[LPTX], x_lds[LPTX];
         bool x_ok[LPTX];
         const int x_dummy = n0 * kH * kW * kGroups;
@@ -240,7 +285,7 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
                 const int f = cell / GB;
                 const int img = f / WPI;
                 const int col = q0 + f % WPI - kPadX;
-                x_lds[l] = g * GSX + f;
+                x_lds[l] = g * GSX + x_image_offset(img) + f % WPI;
                 if (col >= 0 && col < kW && n0 + img < kN && cb * GB + g < kGroups) {
                     x_off[l] = ((n0 + img) * kH * kW + col) * kGroups + cb * GB + g;
                     x_ok[l] = true;
@@ -260,7 +305,7 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
                 const int g = cell % GB;
                 const int q = (cell / GB) % BQ;
                 const int img = cell / (GB * BQ);
-                d_lds[l] = g * GSD + img * WPI + q;
+                d_lds[l] = g * GSD + d_image_offset(img) + q;
                 if (q0 + q < kQ && n0 + img < kN && cb * GB + g < kGroups) {
                     d_off[l] = ((n0 + img) * kP * kQ + q0 + q) * kGroups + cb * GB + g;
                     d_ok[l] = true;
@@ -269,13 +314,21 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
         }
         const spio_uint4 zero4 = spio_uint4{0u, 0u, 0u, 0u};
 
-        // ---- prologue: steps 0..PF-1 into registers, step 0 into LDS ----
+        // ---- prologue: steps S0..S0+PF-1 into registers, step S0 (and the dy rows before it)
+        //      into LDS ----
         spio_uint4 xpre[PF][RB][LPTX], dpre[PF][RB][LPTD];
+        spio_uint4 dlead[LEAD > 0 ? LEAD : 1][LPTD];
+#pragma unroll
+        for (int i = 0; i < LEAD; ++i) {
+            const int pr = imin(p0 + i, kP - 1);
+#pragma unroll
+            for (int l = 0; l < LPTD; ++l) dlead[i][l] = load_stream(dy + d_off[l] + pr * drow_units);
+        }
 #pragma unroll
         for (int sp = 0; sp < PF; ++sp) {
 #pragma unroll
             for (int rr = 0; rr < RB; ++rr) {
-                const int t = sp * RB + rr;
+                const int t = (S0 + sp) * RB + rr;
                 const int h = imin(imax(p0 + t - kPadY, 0), kH - 1);
 #pragma unroll
                 for (int l = 0; l < LPTX; ++l) xpre[sp][rr][l] = load_stream(x + x_off[l] + h * xrow_units);
@@ -292,143 +345,200 @@ SPIO_KERNEL_NAME(float* __restrict__ grad_weight, const spio_uint4* __restrict__
         }
         block_sync();  // rings zeroed / previous image block finished
 #pragma unroll
+        for (int i = 0; i < LEAD; ++i) {
+            const bool drow_ok = i < bh_eff;
+#pragma unroll
+            for (int l = 0; l < LPTD; ++l)
+                if (d_lds[l] >= 0) dring[(i % NRD) * DROW_UNITS + d_lds[l]] = (drow_ok && d_ok[l]) ? dlead[i][l] : zero4;
+        }
+#pragma unroll
         for (int rr = 0; rr < RB; ++rr) {
-            const int h = p0 + rr - kPadY;
+            const int t = S0 * RB + rr;
+            const int h = p0 + t - kPadY;
             const bool xrow_ok = h >= 0 && h < kH;
 #pragma unroll
             for (int l = 0; l < LPTX; ++l)
-                if (x_lds[l] >= 0) xring[rr * XROW_UNITS + x_lds[l]] = (xrow_ok && x_ok[l]) ? xpre[0][rr][l] : zero4;
-            const bool drow_ok = rr < bh_eff;
+                if (x_lds[l] >= 0) xring[((S0 & 1) * RB + rr) * XROW_UNITS + x_lds[l]] = (xrow_ok && x_ok[l]) ? xpre[0][rr][l] : zero4;
+            const bool drow_ok = t < bh_eff;
 #pragma unroll
             for (int l = 0; l < LPTD; ++l)
-                if (d_lds[l] >= 0) dring[rr * DROW_UNITS + d_lds[l]] = (drow_ok && d_ok[l]) ? dpre[0][rr][l] : zero4;
+                if (d_lds[l] >= 0) dring[(t % NRD) * DROW_UNITS + d_lds[l]] = (drow_ok && d_ok[l]) ? dpre[0][rr][l] : zero4;
         }
         block_sync();
 
-        for (int sb = 0; sb < STEPS; sb += PF) {
+        // What step `st` (of parity `sp`) multiplies: x rows t+rr against the aligned dy row pairs
+        // they overlap (x row t+rr and the pair starting at row i2 meet at delta = t + rr - i2).
+        // The row pair starting at tbase is complete in LDS (its second row was staged during
+        // the previous step) when two rows go per step, and on odd steps otherwise; that is
+        // when it is added to the bias sum, once per pair.
+        struct StepPlan {
+            int tbase;
+            bool row_live[RB];
+            bool bias_pair;
+            bool do_math;
+        };
+        auto plan_step = [&](int st, int sp) {
+            StepPlan pl;
+            const int t = st * RB;  // first x row of the step, relative to the block
+            pl.tbase = RB == 2 ? t : t - sp;  // even
+            bool any_live = false;
 #pragma unroll
-            for (int uf = 0; uf < PF; ++uf) {
+            for (int rr = 0; rr < RB; ++rr) {
+                const int hcur = p0 + t + rr - kPadY;
+                pl.row_live[rr] = t + rr < ROWS && hcur >= 0 && hcur < kH;
+                any_live = any_live || pl.row_live[rr];
+            }
+            pl.bias_pair = kDbias && (RB == 2 || sp == 1) && pl.tbase < bh_eff;
+            pl.do_math = wave_active && (any_live || pl.bias_pair);
+            return pl;
+        };
+        // A step's work comes in CPW * NPAIR groups: group (ci, m) is the products of chunk ci with
+        // dy row pair m, and the share m of the chunk's fragment reads (the chunk's RB * NBLK x
+        // fragments and NPAIR dy fragments dealt round-robin over its groups).
+        constexpr int ITEMS = RB * NBLK + NPAIR;  // fragment reads (pairs of LDS reads) per chunk
+        auto read_group = [&](const StepPlan& pl, int sp, int ci, int mslot, spio_half8(&bf)[CPW][RB][NBLK],
+                              spio_half8(&af)[CPW][NPAIR]) {
+            const int ch = ws + TS * ci;
+            if (TS > 1 && ch >= KC) return;
+#pragma unroll
+            for (int j = mslot; j < ITEMS; j += NPAIR) {
+                if (j < RB * NBLK) {
+                    const int rr = j / NBLK, nb = j % NBLK;
+                    const unsigned char* xrow =
+                        reinterpret_cast<const unsigned char*>(xring + (sp * RB + rr) * XROW_UNITS) + xfrag_off;
+                    const unsigned char* pb0 = xrow + (XCP * ch + 2 * nb) * 16;
+                    bf[ci][rr][nb] = read_tr_pair(pb0, pb0 + 4 * 16);
+                } else {
+                    const int m = j - RB * NBLK;
+                    const int i2 = pl.tbase - 2 * m;  // first row of the pair, relative to p0
+                    if (i2 >= 0 && i2 < bh_eff) {
+                        const int slot = (i2 + sel) % NRD;
+                        const unsigned char* pa0 =
+                            reinterpret_cast<const unsigned char*>(dring + slot * DROW_UNITS) + dfrag_off + (32 * ch) * 16;
+                        af[ci][m] = read_tr_pair(pa0, pa0 + 4 * 16);
+                    }
+                }
+            }
+        };
+        auto multiply_group = [&](const StepPlan& pl, int sp, int ci, int m, const spio_half8(&bf)[CPW][RB][NBLK],
+                                  const spio_half8(&af)[CPW][NPAIR]) {
+            const int ch = ws + TS * ci;
+            if (TS > 1 && ch >= KC) return;
+            const int i2 = pl.tbase - 2 * m;
+            if (i2 >= 0 && i2 < bh_eff) {
+#pragma unroll
+                for (int rr = 0; rr < RB; ++rr) {
+                    const int d = (RB == 2 ? rr : sp) + 2 * m;  // = t + rr - i2
+                    if (d <= kR && pl.row_live[rr]) {
+#pragma unroll
+                        for (int nb = 0; nb < NBLK; ++nb)
+                            acc[d][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[ci][m], bf[ci][rr][nb], acc[d][nb],
+                                                                                0, 0, 0);
+                    }
+                }
+                if (m == 0 && pl.bias_pair) accb = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[ci][0], ones8, accb, 0, 0, 0);
+            }
+        };
+        // 2. prefetch step st+PF (its register buffer held step st, now in LDS); rows past the end
+        //    repeat a real row and are never used
+        auto prefetch_rows = [&](int st, int uf) {
+#pragma unroll
+            for (int rr = 0; rr < RB; ++rr) {
+                const int t2 = (st + PF) * RB + rr;
+                const int h = imin(imax(p0 + t2 - kPadY, 0), kH - 1);
+#pragma unroll
+                for (int l = 0; l < LPTX; ++l) xpre[uf % PF][rr][l] = load_stream(x + x_off[l] + h * xrow_units);
+                const int pr = imin(p0 + t2, kP - 1);
+#pragma unroll
+                for (int l = 0; l < LPTD; ++l) dpre[uf % PF][rr][l] = load_stream(dy + d_off[l] + pr * drow_units);
+            }
+        };
+        // 3. the rows of step st+1 into LDS (dy rows past the block's last row become zero).  The
+        //    ring rows written here are not read in this step, except for dy entries whose filter
+        //    row is out of range and whose product is ignored.
+        auto stage_x = [&](int st, int sp, int uf) {
+            if (st + 1 >= S1) return;
+#pragma unroll
+            for (int rr = 0; rr < RB; ++rr) {
+                const int tn = (st + 1) * RB + rr;
+                const int hn = p0 + tn - kPadY;
+                if (tn < ROWS && hn >= 0 && hn < kH) {
+#pragma unroll
+                    for (int l = 0; l < LPTX; ++l)
+                        if (x_lds[l] >= 0)
+                            xring[(((sp + 1) & 1) * RB + rr) * XROW_UNITS + x_lds[l]] =
+                                x_ok[l] ? xpre[(uf + 1) % PF][rr][l] : zero4;
+                }
+            }
+        };
+        auto stage_dy = [&](int st, int uf) {
+            if (st + 1 >= S1) return;
+#pragma unroll
+            for (int rr = 0; rr < RB; ++rr) {
+                const int tn = (st + 1) * RB + rr;
+                const int dslot = tn % NRD;
+                const bool drow_ok = tn < bh_eff;
+#pragma unroll
+                for (int l = 0; l < LPTD; ++l)
+                    if (d_lds[l] >= 0)
+                        dring[dslot * DROW_UNITS + d_lds[l]] = (drow_ok && d_ok[l]) ? dpre[(uf + 1) % PF][rr][l] : zero4;
+            }
+        };
+
+        // With SPIO_PIPE the products of a step are issued one step later, from a second set of
+        // fragment registers, and the step's own LDS reads, row loads and ring writes are dealt
+        // out between the groups of MFMAs: the matrix pipe takes 16 cycles per MFMA and the wave
+        // issues the other instructions in the slots that leaves.  (The compiler does not move
+        // the ring writes, which sit under lane masks, across the MFMAs by itself.)
+        constexpr int FSETS = SPIO_PIPE ? 2 : 1;
+        constexpr int GROUPS = CPW * NPAIR;
+        spio_half8 bfrag[FSETS][CPW][RB][NBLK], afrag[FSETS][CPW][NPAIR];
+        for (int sb = S0; sb < S1; sb += UNROLL) {
+#pragma unroll
+            for (int uf = 0; uf < UNROLL; ++uf) {
                 const int st = sb + uf;
-                if (st >= STEPS) break;
-                const int t = st * RB;  // first x row of the step, relative to the block
+                if (st >= S1) break;
                 // PF is even, so the parity of the step is known at compile time: it fixes the
                 // x ring rows and, with one row per step, the parity of delta.
-                const int sp = uf & 1;
-
-                // 1. read this step's fragments: the x rows t+rr and the aligned dy row pairs
-                //    they overlap (x row t+rr and the pair starting at row i2 meet at
-                //    delta = t + rr - i2).  All LDS reads are issued before anything else so that
-                //    their latency, the global loads and the ring writes below overlap; the
-                //    MFMAs come last.
-                const int tbase = RB == 2 ? t : t - sp;  // even
-                bool row_live[RB];
-                bool any_live = false;
+                const int sp = (S0 + uf) & 1;
+                const StepPlan pl = plan_step(st, sp);
+                if (SPIO_PIPE) {
+                    const int fs = uf & 1;
+                    const StepPlan before = plan_step(st - 1, sp ^ 1);
 #pragma unroll
-                for (int rr = 0; rr < RB; ++rr) {
-                    const int hcur = p0 + t + rr - kPadY;
-                    row_live[rr] = t + rr < ROWS && hcur >= 0 && hcur < kH;
-                    any_live = any_live || row_live[rr];
-                }
-                // The row pair starting at tbase is complete in LDS (its second row was staged
-                // during the previous step) when two rows go per step, and on odd steps otherwise;
-                // that is when it is added to the bias sum, once per pair.
-                const bool bias_pair = kDbias && (RB == 2 || sp == 1) && tbase < bh_eff;
-                const bool do_math = wave_active && (any_live || bias_pair);
-                spio_half8 bfrag[CPW][RB][NBLK], afrag[CPW][NPAIR];
-                if (do_math) {
-#pragma unroll
-                    for (int ci = 0; ci < CPW; ++ci) {
-                        const int ch = ws + TS * ci;
-                        if (TS > 1 && ch >= KC) break;
-#pragma unroll
-                        for (int rr = 0; rr < RB; ++rr) {
-                            const unsigned char* xrow =
-                                reinterpret_cast<const unsigned char*>(xring + (sp * RB + rr) * XROW_UNITS) + xfrag_off;
-#pragma unroll
-                            for (int nb = 0; nb < NBLK; ++nb) {
-                                const unsigned char* pb0 = xrow + (32 * ch + 2 * nb) * 16;
-                                bfrag[ci][rr][nb] = read_tr_pair(pb0, pb0 + 4 * 16);
-                            }
-                        }
-#pragma unroll
-                        for (int m = 0; m < NPAIR; ++m) {
-                            const int i2 = tbase - 2 * m;  // first row of the pair, relative to p0
-                            if (i2 >= 0 && i2 < bh_eff) {
-                                const int slot = (i2 + sel) % NRD;
-                                const unsigned char* pa0 =
-                                    reinterpret_cast<const unsigned char*>(dring + slot * DROW_UNITS) +
-                                    dfrag_off + (32 * ch) * 16;
-                                afrag[ci][m] = read_tr_pair(pa0, pa0 + 4 * 16);
-                            }
-                        }
+                    for (int g = 0; g < GROUPS; ++g) {
+                        const int ci = g / NPAIR, m = g % NPAIR;
+                        if (pl.do_math) read_group(pl, sp, ci, m, bfrag[fs], afrag[fs]);
+                        if (g == 0) prefetch_rows(st, uf);
+                        if (g == (GROUPS > 1 ? 1 : 0)) stage_x(st, sp, uf);
+                        if (g == (GROUPS > 2 ? 2 : GROUPS - 1)) stage_dy(st, uf);
+                        if (st > S0 && before.do_math) multiply_group(before, sp ^ 1, ci, m, bfrag[fs ^ 1], afrag[fs ^ 1]);
+                        __builtin_amdgcn_sched_barrier(0);
                     }
-                }
-
-                // 2. prefetch step st+PF (its register buffer held step st, now in LDS); rows
-                //    past the end repeat a real row and are never used
+                } else {
+                    // all LDS reads first, so that their latency overlaps the loads and ring writes
+                    if (pl.do_math) {
 #pragma unroll
-                for (int rr = 0; rr < RB; ++rr) {
-                    const int t2 = (st + PF) * RB + rr;
-                    const int h = imin(imax(p0 + t2 - kPadY, 0), kH - 1);
-#pragma unroll
-                    for (int l = 0; l < LPTX; ++l) xpre[uf][rr][l] = load_stream(x + x_off[l] + h * xrow_units);
-                    const int pr = imin(p0 + t2, kP - 1);
-#pragma unroll
-                    for (int l = 0; l < LPTD; ++l) dpre[uf][rr][l] = load_stream(dy + d_off[l] + pr * drow_units);
-                }
-
-                // 3. the rows of step st+1 into LDS (dy rows past the block's last row become
-                //    zero).  The ring rows written here are not read in this step, except for dy
-                //    entries whose filter row is out of range and whose product is ignored.
-                if (st + 1 < STEPS) {
-#pragma unroll
-                    for (int rr = 0; rr < RB; ++rr) {
-                        const int tn = t + RB + rr;
-                        const int hn = p0 + tn - kPadY;
-                        if (tn < ROWS && hn >= 0 && hn < kH) {
-#pragma unroll
-                            for (int l = 0; l < LPTX; ++l)
-                                if (x_lds[l] >= 0)
-                                    xring[(((sp + 1) & 1) * RB + rr) * XROW_UNITS + x_lds[l]] =
-                                        x_ok[l] ? xpre[(uf + 1) % PF][rr][l] : zero4;
-                        }
-                        const int dslot = tn % NRD;
-                        const bool drow_ok = tn < bh_eff;
-#pragma unroll
-                        for (int l = 0; l < LPTD; ++l)
-                            if (d_lds[l] >= 0)
-                                dring[dslot * DROW_UNITS + d_lds[l]] =
-                                    (drow_ok && d_ok[l]) ? dpre[(uf + 1) % PF][rr][l] : zero4;
+                        for (int g = 0; g < GROUPS; ++g) read_group(pl, sp, g / NPAIR, g % NPAIR, bfrag[0], afrag[0]);
                     }
-                }
-
-                // 4. multiply
-                if (do_math) {
+                    prefetch_rows(st, uf);
+                    stage_x(st, sp, uf);
+                    stage_dy(st, uf);
+                    if (pl.do_math) {
 #pragma unroll
-                    for (int ci = 0; ci < CPW; ++ci) {
-                        const int ch = ws + TS * ci;
-                        if (TS > 1 && ch >= KC) break;
-#pragma unroll
-                        for (int m = 0; m < NPAIR; ++m) {
-                            const int i2 = tbase - 2 * m;
-                            if (i2 >= 0 && i2 < bh_eff) {
-#pragma unroll
-                                for (int rr = 0; rr < RB; ++rr) {
-                                    const int d = (RB == 2 ? rr : sp) + 2 * m;  // = t + rr - i2
-                                    if (d <= kR && row_live[rr]) {
-#pragma unroll
-                                        for (int nb = 0; nb < NBLK; ++nb)
-                                            acc[d][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                                                afrag[ci][m], bfrag[ci][rr][nb], acc[d][nb], 0, 0, 0);
-                                    }
-                                }
-                                if (m == 0 && bias_pair)
-                                    accb = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[ci][0], ones8, accb, 0, 0, 0);
-                            }
-                        }
+                        for (int g = 0; g < GROUPS; ++g) multiply_group(pl, sp, g / NPAIR, g % NPAIR, bfrag[0], afrag[0]);
                     }
                 }
                 block_sync();
+            }
+        }
+        if (SPIO_PIPE) {
+            constexpr int LAST = S1 - 1;
+            const StepPlan pl = plan_step(LAST, LAST & 1);
+            if (pl.do_math) {
+#pragma unroll
+                for (int g = 0; g < GROUPS; ++g)
+                    multiply_group(pl, LAST & 1, g / NPAIR, g % NPAIR, bfrag[(LAST - S0) & 1], afrag[(LAST - S0) & 1]);
             }
         }
     }

@@ -31,7 +31,7 @@ MAX_LDS_BYTES = 128 * 1024
 MAX_LOADS_PER_THREAD = 8
 MAX_ACCUMULATORS = 32
 MAX_GEOMETRIES = 16
-PIPELINE_CHOICES = ((2, 1), (4, 1), (2, 2))  # (prefetch, rows)
+PIPELINE_CHOICES = ((2, 1, 0), (4, 1, 0), (2, 2, 0), (2, 1, 1), (4, 1, 1))  # (prefetch, rows, pipe)
 
 
 @dataclass(frozen=True)
@@ -56,6 +56,9 @@ class Conv2dGw8WgradConfig:
         variant: "mfma" (row-streaming MFMA kernel) or "direct" (any shape).
         block_q: grad_output columns per workgroup (0: the whole width); the workgroup stages
             block_q + S - 1 columns of x opposite them, so rows of any width fit.
+        pipe: 1 = the MFMAs of a step are issued one step later, from a second set of fragment
+            registers, with the next step's LDS reads, row loads and ring writes dealt out
+            between them; 0 = every step reads its fragments, then multiplies.
     """
 
     groups: int = 8
@@ -69,6 +72,30 @@ class Conv2dGw8WgradConfig:
     split: int = 1
     rows: int = 1
     block_q: int = 0
+    pipe: int = 0
+
+
+def image_placement(params: Conv2dGw8Params, nb: int, block_q: int = 0) -> Dict[str, int]:
+    """Where the images of a staged row sit (mirror of the kernel's constants).
+
+    Images follow one another GAP = max(px, S-1-px) zero cells apart (the right halo of one is
+    the left halo of the next).  The contraction runs over 32-pixel chunks of the grad_output
+    row; where a chunk holds whole images and that takes fewer chunks than the images laid end
+    to end, every chunk gets its own images (PACKED).
+    """
+    s, px = params.s, params.padding_w
+    s2 = 2 * ((s + 1) // 2)
+    bq = block_q or params.q
+    gap = max(px, s - 1 - px)
+    ip = bq + s - 1 if block_q else bq + gap
+    ipc_max = (32 + ip - bq) // ip
+    kc_flat = divup((nb - 1) * ip + bq, 32)
+    kc_packed = divup(nb, ipc_max) if ipc_max > 0 else kc_flat
+    packed = kc_packed < kc_flat
+    kc = kc_packed if packed else kc_flat
+    xcp = 16 * divup(32 + s2 - 1, 16) if packed else 32
+    return dict(IP=ip, IPC=ipc_max if packed else nb, KC=kc, PACKED=int(packed), XCP=xcp,
+                FPX=kc * xcp if packed else 32 * kc + s2 - 1)  # fmt: skip
 
 
 def wgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig) -> Dict[str, int]:
@@ -79,9 +106,8 @@ def wgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig) -> Dic
     bq = config.block_q or params.q
     wpi = bq + s - 1
     f = nb * wpi
-    kspan = (nb - 1) * wpi + bq
-    kc = divup(kspan, 32)
-    fpx = 32 * kc + s2 - 1
+    place = image_placement(params, nb, config.block_q)
+    kc, fpx = place["KC"], place["FPX"]
     gsx = fpx + ((9 - fpx % 16) + 16) % 16
     fpd = 32 * kc
     gsd = fpd + ((9 - fpd % 16) + 16) % 16
@@ -104,7 +130,7 @@ def wgrad_geometry(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig) -> Dic
         GBLKS=divup(params.groups, gb), PBLKS=divup(params.p, bh),
         NBLKS=divup(params.n, nb * iters),
         STEPS=divup(bh + (2 if params.has_bias and r == 1 else r) - 1, rb),
-        PIXEL_EFF=kspan and (nb * bq) / (32.0 * kc),
+        PIXEL_EFF=(nb * bq) / (32.0 * kc), IPC=place["IPC"], PACKED=place["PACKED"],
     )  # fmt: skip
     g["NUM_BLOCKS"] = g["GBLKS"] * g["PBLKS"] * g["QBLKS"] * g["NBLKS"]
     return g
@@ -123,6 +149,7 @@ def _mfma_config_is_legal(params, config) -> bool:
         and config.prefetch >= 2
         and config.prefetch % 2 == 0
         and config.rows in (1, 2)
+        and config.pipe in (0, 1)
         and 0 <= config.block_q <= params.q
         and (g["LPTX"] + g["LPTD"]) * config.prefetch * config.rows <= 32
     )
@@ -164,13 +191,11 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None) -> List[Conv2dGw8Wgr
     # where a padded image row is shorter than a chunk the count decides how full the chunks
     # are: besides the powers of two, the counts that fill them clearly better (7x7 images with
     # one halo column each side: 8 images fill 56 of 96 pixels, 7 images 49 of 64).
-    wpi = params.q + params.s - 1
-
     def chunk_fill(nb):
-        return nb * params.q / (32.0 * divup((nb - 1) * wpi + params.q, 32))
+        return nb * params.q / (32.0 * image_placement(params, nb)["KC"])
 
     image_counts = [1, 2, 4, 8]
-    if wpi < 32:
+    if params.q + params.s - 1 < 32:
         best = max(chunk_fill(nb) for nb in image_counts)
         image_counts += [nb for nb in (3, 5, 6, 7) if chunk_fill(nb) > best + 0.05]
     # Rank the tile geometries first and keep the best few; each of them is then tried with the
@@ -192,10 +217,10 @@ def _get_configs(params: Conv2dGw8Params, device_attr=None) -> List[Conv2dGw8Wgr
     geometries.sort(key=lambda sc: sc[0])
     configs = []
     for _, base in geometries[:MAX_GEOMETRIES]:
-        for pf, rows in PIPELINE_CHOICES:
+        for pf, rows, pipe in PIPELINE_CHOICES:
             if pf > 2 and pf * rows > base.block_h + params.r - 1:
                 continue
-            cfg = replace(base, prefetch=pf, rows=rows)
+            cfg = replace(base, prefetch=pf, rows=rows, pipe=pipe)
             if _mfma_config_is_legal(params, cfg):
                 configs.append(cfg)
     total_pix = params.n * params.p * params.q
@@ -223,6 +248,8 @@ def _get_kernel_spec(params: Conv2dGw8Params, config: Conv2dGw8WgradConfig, _dev
     defines.update(SPIO_GB=config.groups, SPIO_BH=config.block_h, SPIO_NB=config.block_n,
                    SPIO_ITERS=config.block_n_iters, SPIO_PF=config.prefetch,
                    SPIO_TS=config.split, SPIO_RB=config.rows)  # fmt: skip
+    if config.pipe:
+        defines["SPIO_PIPE"] = 1
     if config.block_q:
         defines["SPIO_BQ"] = config.block_q
     spec = KernelSpec(defines, LaunchParams(grid=g["NUM_BLOCKS"], block=g["THREADS"]), MFMA_SOURCE, notes=g)

@@ -142,6 +142,41 @@ def test_column_blocks_weight_gradient_and_fused_backward():
         run_bgrad_kernel_test(conv2d_gw8_bgrad_kernel_factory, params, configs=bconfigs)
 
 
+def test_weight_gradient_packed_images_skipped_padding_and_pipeline():
+    """Small images under large filters: images sharing their halo columns, chunks that hold their
+    own images (14x14 under 7x7: two per 32-pixel chunk; 10 wide under 3x3: three), whole-image
+    workgroups that skip the steps whose x rows are padding (odd and even first step, one and two
+    rows per step; not with a bias), and the pipelined step (MFMAs one step behind the reads) with
+    atomics, two stages, split groups, ragged batches and ragged channel blocks."""
+    W = Conv2dGw8WgradConfig
+    cases = [
+        (Conv2dGw8Params(n=10, c=32, h=14, w=14, r=7, s=7, padding=3, has_bias=False),
+         [W(groups=4, block_h=14, block_n=4, block_n_iters=2, prefetch=4, two_stage=1),
+          W(groups=4, block_h=14, block_n=4, block_n_iters=2, prefetch=4, two_stage=1, pipe=1),
+          W(groups=4, block_h=14, block_n=8, prefetch=2, pipe=1),
+          W(groups=4, block_h=14, block_n=6, prefetch=2, two_stage=1, split=3, pipe=1),
+          W(groups=2, block_h=14, block_n=4, prefetch=2, rows=2, pipe=1),
+          W(groups=4, block_h=14, block_n=4, prefetch=2, rows=2, two_stage=1),
+          W(groups=4, block_h=7, block_n=4, prefetch=2, pipe=1)]),
+        (Conv2dGw8Params(n=7, c=24, h=14, w=14, r=7, s=7, padding=3, has_bias=True),
+         [W(groups=3, block_h=14, block_n=4, prefetch=2, pipe=1), W(groups=2, block_h=14, block_n=4, prefetch=4, two_stage=1)]),
+        (Conv2dGw8Params(n=13, c=16, h=9, w=10, padding=1, has_bias=False),
+         [W(groups=2, block_h=9, block_n=6, prefetch=2), W(groups=2, block_h=9, block_n=6, prefetch=2, pipe=1),
+          W(groups=2, block_h=9, block_n=3, block_n_iters=2, prefetch=4, pipe=1, two_stage=1)]),
+        (Conv2dGw8Params(n=9, c=16, h=12, w=15, r=5, s=5, padding=2, has_bias=False),
+         [W(groups=2, block_h=12, block_n=4, prefetch=2, pipe=1), W(groups=2, block_h=12, block_n=4, prefetch=2, rows=2, pipe=1),
+          W(groups=2, block_h=12, block_n=2, prefetch=4)]),
+        (Conv2dGw8Params(n=5, c=16, h=11, w=13, r=4, s=6, padding=(1, 4), has_bias=False),
+         [W(groups=2, block_h=9, block_n=4, prefetch=2, pipe=1), W(groups=2, block_h=9, block_n=2, prefetch=2)]),
+        (Conv2dGw8Params(n=6, c=64, h=56, w=56, padding=1, has_bias=False),
+         [W(groups=4, block_h=56, prefetch=2, rows=2, pipe=1), W(groups=8, block_h=56, prefetch=4, pipe=1, block_n_iters=2)]),
+        (Conv2dGw8Params(n=16, c=48, h=7, w=7, padding=1, has_bias=True),
+         [W(groups=6, block_h=7, block_n=8, prefetch=2, pipe=1), W(groups=6, block_h=7, block_n=4, block_n_iters=2, prefetch=2)]),
+    ]  # fmt: skip
+    for params, configs in cases:
+        run_grad_kernel_test(conv2d_gw8_wgrad_kernel_factory, params, configs=configs)
+
+
 # shapes the fused backward kernel has a configuration for: any padding, odd and even filter
 # sizes (7x7 needs more registers than a wave has and stays with the separate kernels)
 FUSED = [p for p in SANITY if bgrad_is_supported(p) and list(conv2d_gw8_bgrad_kernel_factory.configs(p))] + [
