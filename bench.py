@@ -263,8 +263,24 @@ def copy_ceiling(nbytes, device, iters):
         us = run(fn, grid, threads, lambda d, s, g=grid: (d, s, n, g))
         variants.append({"kernel": "spio_stream_copy_strided", "threads": threads, "unroll": unroll,
                          "grid": grid, "us": round(us, 2), "GB/s": round(2 * n * 16 / us / 1e3, 1)})  # fmt: skip
-    del sets
+    # two tensors in, one out: the fused backward kernel's mix (every set gets a second source of
+    # its own, so that no launch reads what its predecessor has just read)
+    second = {id(s): torch.randint(0, 2**31 - 1, (n * 4,), dtype=torch.int32, device=device) for _d, s in sets}
+    combine = []
+    for threads, unroll, mult in ((512, 1, 16), (256, 2, 16), (256, 4, 8), (512, 2, 8)):
+        chunks = n // (threads * unroll)
+        if chunks == 0:
+            continue
+        grid = min(chunks, cus * mult)
+        defines = {"SPIO_COPY_THREADS": threads, "SPIO_COPY_UNROLL": unroll}
+        m, fn = compile_and_load_kernel("spio_stream_combine_strided", "stream_copy.hip", defines, device.index or 0)
+        keep.append(m)
+        us = run(fn, grid, threads, lambda d, s, g=grid: (d, s, second[id(s)], n, g))
+        combine.append({"kernel": "spio_stream_combine_strided", "threads": threads, "unroll": unroll,
+                        "grid": grid, "us": round(us, 2), "GB/s": round(3 * n * 16 / us / 1e3, 1)})  # fmt: skip
+    del sets, second
     best = max(variants, key=lambda v: v["GB/s"])
+    best2 = max(combine, key=lambda v: v["GB/s"]) if combine else None
     return {
         "bytes": 2 * n * 16,
         "buffer_sets": nsets,
@@ -272,6 +288,9 @@ def copy_ceiling(nbytes, device, iters):
         "plain": variants[0],
         "frac_of_hbm_peak": round(best["GB/s"] / HBM_PEAK_GBS, 4),
         "variants": variants,
+        "two_in_one_out": {"bytes": 3 * n * 16, "best": best2, "variants": combine,
+                           "note": "dst = a ^ b over three tensors of the same size: the HBM rate a kernel that "
+                                   "reads two activation tensors and writes one reaches (the fused backward's mix)"},
         "note": "non-temporal copies of one activation tensor in and one out over rotating buffers: "
                 "the HBM rate a read-X/write-X kernel reaches on this device",
     }
@@ -632,6 +651,9 @@ def bench_conv(args, device, workload=None, full=True):
     result["copy_ceiling"] = copy_ceiling(act_bytes, device, iters)
     best = result["copy_ceiling"]["best"]["GB/s"]
     result["roofline"]["frac_of_copy_ceiling"] = round(kernels[dominant]["GB/s"] / best, 4)
+    two_one = result["copy_ceiling"]["two_in_one_out"]["best"]
+    if two_one and "bgrad" in kernels:
+        result["bgrad_frac_of_two_in_one_out_stream"] = round(kernels["bgrad"]["GB/s"] / two_one["GB/s"], 4)
     result["fprop_frac_of_copy_ceiling"] = round(kernels["fprop"]["GB/s"] / best, 4)
     if not args.no_cpu_baseline:
         torch.cuda.empty_cache()
