@@ -71,6 +71,16 @@ WORKLOADS = {
 SWEEP_BATCHES = (1, 2, 4, 8, 16, 32, 64, 128, 256, 512)
 NETWORK_WIDTHS = ((96, 56), (192, 28), (384, 14), (768, 7))
 LAUNCH_FLOOR_US = 2.2  # an empty kernel in the same back-to-back loop
+# What a plain streaming kernel needs for a given volume on this device: the launch floor plus the
+# bytes at the marginal rate of the copy kernels (their time against size is a fixed 1.5-2.4 us
+# plus 6.0-6.4 TB/s).  `frac_of_stream_model` = that time / the kernel's: a kernel near 1 has
+# nothing left but the launch floor and the bytes, whatever its share of the 8 TB/s peak is.
+STREAM_RATE_GBS = 6200.0
+
+
+def stream_model(us, nbytes):
+    model = LAUNCH_FLOOR_US + nbytes / (STREAM_RATE_GBS * 1e3)
+    return {"stream_model_us": round(model, 2), "frac_of_stream_model": round(model / us, 3)}
 
 
 def parse_args():
@@ -568,6 +578,7 @@ def bench_conv(args, device, workload=None, full=True):
         attach_profile_figures(kernels[name], workload, name)
         # what an empty kernel costs in the same back-to-back loop, as a share of this kernel's time
         kernels[name]["launch_floor_share"] = round(LAUNCH_FLOOR_US / kernels[name]["us"], 3)
+        kernels[name].update(stream_model(kernels[name]["us"], kernels[name]["bytes"]))
     roofline = {
         "bound": "hbm",
         "kernel": kernels[dominant]["kernel"],
@@ -586,7 +597,7 @@ def bench_conv(args, device, workload=None, full=True):
         compact = {}
         for name, e in kernels.items():
             compact[name] = {k: e[k] for k in ("us", "us_min", "GB/s", "frac_of_hbm_peak", "traffic", "traffic_stale",
-                                               "mfma_util", "launch_floor_share", "bytes") if k in e}
+                                               "mfma_util", "launch_floor_share", "frac_of_stream_model", "bytes") if k in e}
             compact[name]["config"] = {k: v for k, v in e["config"].items() if v not in (0, None)}
         return {
             "workload": desc, "params": params.encode(), "step_kernels": in_step,
@@ -692,7 +703,8 @@ def bench_batch_sweep(args, device, full=True):
         e = kernel_entry(k_fwd, [(s["y"], s["x"], w, None) for s in sets], fb, iters, min_seconds)
         point = {"N": n, "fprop_us": e["us"], "fprop_GB/s": e["GB/s"], "fprop_frac": e["frac_of_hbm_peak"],
                  "fprop_bytes": fb, "launch_floor_dominated": e["us"] < 3 * LAUNCH_FLOOR_US,
-                 "fprop_launch_floor_share": round(LAUNCH_FLOOR_US / e["us"], 3)}  # fmt: skip
+                 "fprop_launch_floor_share": round(LAUNCH_FLOOR_US / e["us"], 3),
+                 "fprop_frac_of_stream_model": stream_model(e["us"], fb)["frac_of_stream_model"]}  # fmt: skip
         k_fused = fused_backward_kernel(params, device)
         st_w = Conv2dStats(params, output_names="grad_weight")
         wb = st_w.bytes_read + st_w.grad_weight_bytes_written_fp32
@@ -793,7 +805,7 @@ def bench_network(args, device, full=True):
         e["launch_floor_share"] = round(LAUNCH_FLOOR_US / e["us"], 3)
         convs.append({"shape": params.encode(), "count": depth[c], "us": e["us"], "GB/s": e["GB/s"],
                       "frac_of_hbm_peak": e["frac_of_hbm_peak"], "bytes": nb,
-                      "launch_floor_share": e["launch_floor_share"]})  # fmt: skip
+                      "launch_floor_share": e["launch_floor_share"], **stream_model(e["us"], nb)})  # fmt: skip
         total_bytes += depth[c] * nb
         total_us += depth[c] * e["us"]
         del asets

@@ -323,3 +323,44 @@ def test_fused_backward_works_on_the_larger_of_input_and_output():
     assert bgrad_domain(even) == (29, 28) and bgrad_geometry(even, cfg)["STEPS"] == 7 + 1 + 3
     assert bgrad_domain(Conv2dGw8Params(n=4, c=32, h=28, w=28, r=4, s=4, padding=(0, 3))) == (28, 31)
     assert all(bgrad_is_supported(p) for p in (same, small, large, even))
+
+
+def test_weight_gradient_image_placement_reads_the_right_pixels():
+    """The staged-row layout of the weight-gradient kernel (images sharing halo columns, chunks
+    that hold their own images), restated from its constants: for every grad_output pixel and
+    column tap, the x cell the contraction reads is that image's own column, or a cell no image
+    ever writes (zero) where the column lies in the padding."""
+    from spio_amd.kernels.conv2d_gw8_wgrad_kernel import image_placement
+
+    cases = [(14, 7, 3, (1, 2, 3, 4, 5, 6, 8)), (14, 3, 1, (2, 4, 8)), (7, 3, 1, (4, 7, 8)), (10, 3, 1, (3, 6)),
+             (15, 5, 2, (2, 4)), (13, 6, 4, (2, 4)), (28, 3, 1, (1, 2)), (9, 5, 0, (3, 5)), (12, 4, 3, (2, 4))]
+    packed_seen = False
+    for w, s, px, counts in cases:
+        params = Conv2dGw8Params(n=8, c=16, h=w, w=w, r=1, s=s, padding=(0, px))
+        q_width = params.q
+        for nb in counts:
+            g = image_placement(params, nb)
+            ip, ipc, kc, xcp = g["IP"], g["IPC"], g["KC"], g["XCP"]
+            packed_seen |= bool(g["PACKED"])
+            d_off = [(i // ipc) * 32 + (i % ipc) * ip for i in range(nb)]
+            x_off = [(i // ipc) * xcp + (i % ipc) * ip for i in range(nb)]
+            assert max(d_off) + q_width <= 32 * kc
+            assert kc <= (((nb - 1) * (q_width + s - 1) + q_width) + 31) // 32  # never more chunks than before
+            owner = {}  # x cell -> (image, column) of the data it holds
+            for i in range(nb):
+                for col in range(params.w):
+                    cell = x_off[i] + col + px
+                    assert cell not in owner and cell < g["FPX"]
+                    owner[cell] = (i, col)
+            for i in range(nb):
+                for q in range(q_width):
+                    pos = d_off[i] + q
+                    chunk, local = divmod(pos, 32)
+                    for tap in range(s):
+                        cell = chunk * xcp + local + tap  # what the B fragment of this tap reads
+                        col = q + tap - px
+                        if 0 <= col < params.w:
+                            assert owner.get(cell) == (i, col), (w, s, px, nb, i, q, tap)
+                        else:
+                            assert cell not in owner, (w, s, px, nb, i, q, tap)
+    assert packed_seen
