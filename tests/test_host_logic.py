@@ -364,3 +364,31 @@ def test_weight_gradient_image_placement_reads_the_right_pixels():
                         else:
                             assert cell not in owner, (w, s, px, nb, i, q, tap)
     assert packed_seen
+
+
+def test_counter_figures_in_profiles_were_measured_with_the_committed_kernel_sources():
+    """bench.py reads roofline.traffic and mfma_util from profiles/*.md; every such line names the
+    kernel source and the digest of the text it was measured with.  A kernel edited after its
+    profile was taken would make bench.py report traffic_stale: the committed state has none."""
+    import importlib.util
+    import re
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("bench_module", os.path.join(root, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    seen = 0
+    for workload in ("target", "cfg1", "cfg2", "cfg3"):
+        for kernel in ("fprop", "dgrad", "wgrad", "bgrad"):
+            for kind in ("traffic_bytes", "mfma_util"):
+                value, stale = bench.profile_figure(kind, workload, kernel)
+                if value is None:
+                    assert (workload, kernel) == ("cfg3", "bgrad")  # 7x7 has no fused backward kernel
+                    continue
+                assert stale is False, (kind, workload, kernel)
+                seen += 1
+    assert seen == 30
+    # the model bench.py prices every kernel against: launch floor + bytes at the copy's marginal rate
+    m = bench.stream_model(18.3, 102769664)
+    assert abs(m["stream_model_us"] - (2.2 + 102769664 / 6.2e6)) < 0.01 and 0.9 < m["frac_of_stream_model"] < 1.1
+    assert re.fullmatch(r"[0-9a-f]{12}", bench.source_digest("conv2d_gw8_mfma.hip"))
