@@ -219,8 +219,8 @@ SPIO_KERNEL_NAME(float* __restrict__ partials, ln_uint4* __restrict__ din, const
 }
 
 // Second stage: sums[i] = sum over the workgroups' rows of partials[row][i], i < 2*C.  A workgroup
-// owns 32 columns; its 8 slices each add the rows r = slice, slice + 8, ... with 8 loads in
-// flight, and meet in LDS.  Every element has one owner: no atomics, no dependence on timing.
+// owns 32 columns; its 8 slices each add the rows r = slice, slice + 8, ... with up to 32 loads
+// in flight, and meet in LDS.  Every element has one owner: no atomics, no dependence on timing.
 #define SPIO_LN_CONCAT2(a, b) a##b
 #define SPIO_LN_CONCAT(a, b) SPIO_LN_CONCAT2(a, b)
 extern "C" __global__ void __attribute__((amdgpu_flat_work_group_size(256, 256)))
@@ -228,7 +228,9 @@ SPIO_LN_CONCAT(SPIO_KERNEL_NAME, _reduce)(float* __restrict__ sums, const float*
     constexpr int ROWS = SPIO_LN_GRID;
     constexpr int COLS = 32;
     constexpr int SLICES = 256 / COLS;
-    constexpr int UNR = 8;
+    // as many rows in flight per thread as a slice has, up to 32: one round trip to memory for up
+    // to 256 rows (with 8 in flight the stage took 1.5-2 us longer on the 7x7 and 14x14 shapes)
+    constexpr int UNR = (ROWS + SLICES - 1) / SLICES < 32 ? (ROWS + SLICES - 1) / SLICES : 32;
     __shared__ float red[SLICES][COLS];
     const int tid = (int)__builtin_amdgcn_workitem_id_x();
     const int cl = tid % COLS;
