@@ -71,6 +71,7 @@ WORKLOADS = {
 SWEEP_BATCHES = (1, 2, 4, 8, 16, 32, 64, 128, 256, 512)
 NETWORK_WIDTHS = ((96, 56), (192, 28), (384, 14), (768, 7))
 LAUNCH_FLOOR_US = 2.2  # an empty kernel in the same back-to-back loop
+WARM_SECONDS = 0.03  # of back-to-back launches before a kernel is timed
 # What a plain streaming kernel needs for a given volume on this device: the launch floor plus the
 # bytes at the marginal rate of the copy kernels (their time against size is a fixed 1.5-2.4 us
 # plus 6.0-6.4 TB/s).  `frac_of_stream_model` = that time / the kernel's: a kernel near 1 has
@@ -176,7 +177,11 @@ def timed_blocks(run_block, min_seconds=MIN_TIMED_SECONDS, max_blocks=400):
 
 def time_kernel(kernel, arg_sets, iters, min_seconds=MIN_TIMED_SECONDS):
     """Median and min microseconds per call over repeated event-timed blocks of `iters` launches."""
-    kernel.time(arg_sets, warmup=10, iters=iters)
+    # warm-up: the first tens of milliseconds after a pause (new buffers, another kernel's set-up)
+    # read up to 5 % slow
+    warm = 0.0
+    while warm < WARM_SECONDS:
+        warm += kernel.time(arg_sets, warmup=10, iters=iters) * 1e-3 * iters
     per_call = []
     total = 0.0
     while (total < min_seconds or len(per_call) < 3) and len(per_call) < 400:
