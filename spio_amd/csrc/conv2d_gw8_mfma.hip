@@ -113,6 +113,12 @@ constexpr int WAVES = GB * TS;
 constexpr int THREADS = 64 * WAVES;
 
 constexpr int NS = 2 * ((kR + 1) / 2);  // accumulator row slots
+// With an odd filter height every slot rests for one step between two output rows: the finished
+// row can then be converted and staged one step after its last tap (see the step loop).
+#ifndef SPIO_LATE_EMIT
+#define SPIO_LATE_EMIT 1
+#endif
+constexpr bool kLateEmit = SPIO_LATE_EMIT && NS > kR;
 constexpr int NACC = NS / 2;            // accumulators (pairs of slots) per tile
 constexpr int KB = (kS + 3) / 4;        // MFMA K-steps per source row (4 column taps each)
 // Column blocks (SPIO_BQ > 0): a workgroup owns BQ output columns of its rows and stages the
@@ -484,64 +490,78 @@ SPIO_DEVICE void conv_rows(spio_uint4* __restrict__ dst, const spio_uint4* __res
             }
         }
     };
+    // Stages the output row that received its last tap at step `te` (stage buffer te mod 2) and
+    // resets its slot to the bias.  The row sits in one half of the lanes (slot j = lane / 32).
+    // (Letting the other half convert along and write into spare bytes, which removes the
+    // lane-dependent branch, is slower: 1-6 % at the benchmark shapes.)
+    auto emit_row = [&](int te) {
+        const int slot = pmod(te % NS - (kR - 1), NS);
+        const int a = slot >> 1;
+        const int j = slot & 1;
+        if (out_j == j) {
+#pragma unroll
+            for (int i = 0; i < TPW; ++i) {
+                const int tile = ws + TS * i;
+                if (TS == 1 || tile < WT) {
+                    if (te >= kR - 1) {
+                        Pack8 o;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) o.h[e] = (spio_half)acc[i][a][e];
+                        typedef __attribute__((address_space(3))) spio_uint2* lds_u2p;
+                        *(lds_u2p)(ostage_lane + (te & 1) * OUT_ROW_BYTES + 16 * TS * i * OSTRIDE) = o.u;
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[i][a][e] = bias_reg[e];
+                }
+            }
+        }
+    };
+    auto multiply_tile = [&](int ph, int i) {
+        const int tile = ws + TS * i;
+        if (TS == 1 || tile < WT) {
+#pragma unroll
+            for (int a = 0; a < NACC; ++a) {
+                const int d = pmod(ph - 2 * a, NS);
+#pragma unroll
+                for (int u = 0; u < KB; ++u)
+                    acc[i][a] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wfrag[d][u], bfrag[i][u], acc[i][a], 0, 0, 0);
+            }
+        }
+    };
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) {
         const int ph = t % NS;    // all of these are compile-time constants after unrolling
-        const int obuf = t & 1;   // output stage buffer of this step
 
         // 1. prefetch the next source rows, at most up to row t+PF (whose register buffer is
         //    free: row t is in LDS)
 #pragma unroll
         for (int r = rows_requested(t - 1, STEPS); r < rows_requested(t, STEPS); ++r) load_row(pre[r % PF], r);
 
-        // 2. fragment reads of this step's row; the previous step's output row is stored while
-        //    they are in flight
+        // 2. fragment reads of this step's row; a finished output row is stored while they are
+        //    in flight
         const bool row_live = row_is_live(t);
         if (row_live) read_fragments(bfrag, t % NR);
-        if (t >= kR) store_output_row(t - 1, (t + 1) & 1);
-
+        if (kLateEmit) {
+            // The row that received its last tap in the previous step is converted and staged
+            // now, ahead of this step's multiplications: its results are long complete, and the
+            // conversion runs while the fragment reads are on their way instead of behind the
+            // MFMAs it would have to wait for.  Its slot rests during this step (NS > R: the
+            // slot's filter row is out of range, its A rows are zero), so the values are still
+            // there, and the reset takes effect before the slot's next row begins.  The row
+            // staged in the previous step goes out.
+            if (t >= kR + 1) store_output_row(t - 2, t & 1);
+            if (t >= 1) emit_row(t - 1);  // (before the first finished row: resets only)
+        } else {
+            if (t >= kR) store_output_row(t - 1, (t + 1) & 1);
+        }
         // 3. multiply source row t into the live output rows
         if (row_live) {
 #pragma unroll
-            for (int i = 0; i < TPW; ++i) {
-                const int tile = ws + TS * i;
-                if (TS == 1 || tile < WT) {
-#pragma unroll
-                    for (int a = 0; a < NACC; ++a) {
-                        const int d = pmod(ph - 2 * a, NS);
-#pragma unroll
-                        for (int u = 0; u < KB; ++u)
-                            acc[i][a] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                                wfrag[d][u], bfrag[i][u], acc[i][a], 0, 0, 0);
-                    }
-                }
-            }
+            for (int i = 0; i < TPW; ++i) multiply_tile(ph, i);
         }
 
         // 4. the row that received its last tap: stage it, reset its slot
-        {
-            const int slot = pmod(ph - (kR - 1), NS);
-            const int a = slot >> 1;
-            const int j = slot & 1;
-            const bool emit = t >= kR - 1;
-            if (out_j == j) {
-#pragma unroll
-                for (int i = 0; i < TPW; ++i) {
-                    const int tile = ws + TS * i;
-                    if (TS == 1 || tile < WT) {
-                        if (emit) {
-                            Pack8 o;
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) o.h[e] = (spio_half)acc[i][a][e];
-                            typedef __attribute__((address_space(3))) spio_uint2* lds_u2p;
-                            *(lds_u2p)(ostage_lane + obuf * OUT_ROW_BYTES + 16 * TS * i * OSTRIDE) = o.u;
-                        }
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) acc[i][a][e] = bias_reg[e];
-                    }
-                }
-            }
-        }
+        if (!kLateEmit) emit_row(t);
 
         // 5. the next source row not yet in the ring (loaded earlier) into its ring row
         if (t + 1 < STEPS) {
@@ -550,6 +570,12 @@ SPIO_DEVICE void conv_rows(spio_uint4* __restrict__ dst, const spio_uint4* __res
                 ring[((t + 1) % NR) * RING_ROW_UNITS + in_lds[l]] = pre[(t + 1) % PF][l];
         }
 
+        block_sync();
+    }
+    if (kLateEmit) {
+        // the row staged in the last step goes out, the last row is staged and follows
+        if (STEPS >= kR + 1) store_output_row(STEPS - 2, STEPS & 1);
+        emit_row(STEPS - 1);
         block_sync();
     }
     store_output_row(STEPS - 1, (STEPS - 1) & 1);  // the last row
