@@ -79,6 +79,28 @@ def sample_params(seed: int, count: int = MAX_TEST_PARAMS) -> List[Conv2dGw8Para
     return random.Random(seed).sample(pool, count)
 
 
+def random_params(seed: int, count: int, max_elements: int = 3_000_000) -> List[Conv2dGw8Params]:
+    """Seeded random shapes beyond the reference's list: every filter size from 1x1 to 7x7 with
+    r != s, padding from none to more than the filter's half, odd image sizes and batches, few
+    and many groups.  Sizes stay small enough for the CPU oracle."""
+    rng = random.Random(seed)
+    out = []
+    while len(out) < count:
+        r, s = rng.randint(1, 7), rng.randint(1, 7)
+        if rng.random() < 0.3:
+            r = s = rng.choice([3, 3, 5, 7])
+        py = rng.choice([r // 2, r // 2, 0, rng.randint(0, r)])
+        px = rng.choice([s // 2, s // 2, 0, rng.randint(0, s)])
+        h = rng.choice([rng.randint(1, 20), rng.randint(1, 70), 7, 14, 28, 56])
+        w = rng.choice([rng.randint(1, 20), rng.randint(1, 70), 7, 14, 28, 56, 33, 65, 96])
+        n = rng.choice([1, 2, 3, 5, 8, rng.randint(1, 9)])
+        c = 8 * rng.choice([1, 2, 3, 4, 5, 8, 12, 16, rng.randint(1, 24)])
+        params = Conv2dGw8Params(n=n, c=c, h=h, w=w, r=r, s=s, padding=(py, px), has_bias=rng.random() < 0.5)
+        if params.is_valid() and n * c * max(h * w, params.p * params.q) <= max_elements:
+            out.append(params)
+    return out
+
+
 def pick_configs(factory, params, device_attr, configs=None, limit=MAX_TEST_CONFIGS, seed=0, **kw):
     """All given configs, or a bounded spread of the legal ones (first, last, random)."""
     if configs is not None:
