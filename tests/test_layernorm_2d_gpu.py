@@ -5,6 +5,8 @@ statistics over C per pixel); the reference has no test for it, so torch is the 
 Tolerance: one fp16 rounding of an O(1..10) value plus fp32 statistics: rtol 2e-3, atol 4e-3.
 """
 
+import os
+
 import pytest
 import torch
 import torch.nn.functional as F
@@ -128,6 +130,74 @@ def test_every_backward_configuration_of_one_shape():
         sums = sums.cpu()
         torch.testing.assert_close(sums[0], ex_dw, rtol=2e-3, atol=3e-2, msg=str(config))
         torch.testing.assert_close(sums[1], ex_db, rtol=2e-3, atol=3e-2, msg=str(config))
+        kernel.unload()
+
+
+def _random_layernorm_params(seed, count):
+    import random
+
+    rng = random.Random(seed)
+    out = []
+    while len(out) < count:
+        c = 8 * rng.choice([1, 2, 3, 5, 8, 12, 24, 48, 96, 128, rng.randint(1, 128)])
+        n, h, w = rng.randint(1, 9), rng.choice([1, 7, 14, rng.randint(1, 40)]), rng.choice([1, 7, 14, rng.randint(1, 40)])
+        if n * c * h * w <= 2_000_000:
+            out.append(LayerNorm2dParams(n=n, c=c, h=h, w=w, has_weight=rng.random() < 0.7, has_bias=rng.random() < 0.5,
+                                         eps=rng.choice([1e-6, 1e-5, 1e-3])))  # fmt: skip
+    return out
+
+
+_RANDOM_LN = _random_layernorm_params(int(os.environ.get("SPIO_RANDOM_SEED", "7")),
+                                      int(os.environ.get("SPIO_RANDOM_LAYERNORMS", "6")))  # fmt: skip
+
+
+@pytest.mark.parametrize("params", _RANDOM_LN, ids=lambda p: p.encode())
+def test_random_shapes_every_configuration_forward_and_backward(params):
+    """Seeded random shapes (channel counts 8..1024 that are not powers of two, pixel counts that
+    leave ragged passes, with and without weight and bias, three eps values): every legal
+    configuration of the forward kernel and, where the shape has one, of the backward kernel."""
+    attr = get_device_attributes(0)
+    g = torch.Generator().manual_seed(params.n + params.c + params.h + params.w)
+    x = (torch.randn(params.shape, generator=g) * 2 + 0.5).half()
+    dy = torch.randn(params.shape, generator=g).half()
+    w = torch.randn(params.c, generator=g) if params.has_weight else None
+    b = torch.randn(params.c, generator=g) if params.has_bias else None
+    expected = _reference(x, w, b, params.eps)
+    xg = x.cuda().contiguous(memory_format=torch.channels_last)
+    dyg = dy.cuda().contiguous(memory_format=torch.channels_last)
+    wg = None if w is None else w.cuda()
+    bg = None if b is None else b.cuda()
+    for config in layernorm_2d_kernel_factory.configs(params, attr):
+        kernel = layernorm_2d_kernel_factory.make_kernel(params, config, attr)
+        kernel.compile()
+        kernel.load(0)
+        out = torch.full_like(xg, -42.0)
+        kernel(out, xg, wg, bg)
+        torch.cuda.synchronize()
+        torch.testing.assert_close(out.float().cpu(), expected, rtol=2e-3, atol=4e-3, msg=f"{params.encode()} {config}")
+        kernel.unload()
+    from dataclasses import replace
+
+    params = replace(params, has_bias=False)  # the backward kernel never sees the bias
+    if not layernorm_2d_bwd_is_supported(params):
+        return
+    ex_dx, ex_dw, _ = _reference_backward(x, dy, w, None, params.eps)
+    ex_db = dy.float().sum(dim=(0, 2, 3))
+    if ex_dw is None:
+        ex_dw = (dy.float() * _reference(x, None, None, params.eps)).sum(dim=(0, 2, 3))
+    for config in layernorm_2d_bwd_kernel_factory.configs(params, attr):
+        kernel = layernorm_2d_bwd_kernel_factory.make_kernel(params, config, attr)
+        kernel.compile()
+        kernel.load(0)
+        dx = torch.full_like(xg, -42.0)
+        sums = torch.full((2, params.c), float("nan"), device="cuda")
+        kernel(sums, dx, xg, dyg, wg)
+        torch.cuda.synchronize()
+        what = f"{params.encode()} {config}"
+        torch.testing.assert_close(dx.float().cpu(), ex_dx, rtol=4e-3, atol=4e-3, msg=what)
+        sums = sums.cpu()
+        torch.testing.assert_close(sums[0], ex_dw, rtol=2e-3, atol=3e-2, msg=what)
+        torch.testing.assert_close(sums[1], ex_db, rtol=2e-3, atol=3e-2, msg=what)
         kernel.unload()
 
 
