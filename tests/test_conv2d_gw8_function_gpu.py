@@ -7,11 +7,13 @@ implementation runs, gradients come from torch.autograd.grad, and everything is
 compared with the fp32 CPU oracle.
 """
 
+import os
+
 import pytest
 import torch
 from torch import nn
 
-from helpers import sample_params, to_gpu
+from helpers import random_params, sample_params, to_gpu
 from oracle import conv2d_gw8_oracle as oracle
 from spio_amd.functional import conv2d_gw8
 from spio_amd.kernels import Conv2dGw8Params, Conv2dStats
@@ -86,6 +88,18 @@ def test_function_grad(params):
 def test_function_sampled(params):
     run_function_test(params, seed=1)
     run_grad_function_test(params, seed=1)
+
+
+_RANDOM = random_params(int(os.environ.get("SPIO_RANDOM_SEED", "7")) + 100,
+                        int(os.environ.get("SPIO_RANDOM_FUNCTION_SHAPES", "6")))  # fmt: skip
+
+
+@pytest.mark.parametrize("params", _RANDOM, ids=lambda p: p.encode())
+def test_function_random_shapes(params):
+    """The operator and its autograd on seeded random shapes outside the reference's list (the
+    kernels and tile configurations the operator itself selects, fused or separate backward)."""
+    run_function_test(params, seed=2)
+    run_grad_function_test(params, seed=2)
 
 
 def test_backward_op_skips_what_is_not_needed():
