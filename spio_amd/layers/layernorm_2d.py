@@ -16,7 +16,7 @@ class LayerNorm2d(nn.LayerNorm):
     """
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:  # pylint: disable=arguments-renamed
-        dtype = torch.get_autocast_gpu_dtype() if torch.is_autocast_enabled() else x.dtype
+        dtype = torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled("cuda") else x.dtype
         if (x.is_cuda and x.dim() == 4 and dtype == torch.float16 and x.shape[1] % 8 == 0
                 and len(self.normalized_shape) == 1 and x.shape[1] <= 2048):  # fmt: skip
             return layernorm_2d(x.to(torch.float16), self.weight, self.bias, self.eps).to(x.dtype)
