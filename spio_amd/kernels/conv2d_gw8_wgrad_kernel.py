@@ -152,6 +152,8 @@ def _mfma_config_is_legal(params, config) -> bool:
         and config.pipe in (0, 1)
         and 0 <= config.block_q <= params.q
         and (g["LPTX"] + g["LPTD"]) * config.prefetch * config.rows <= 32
+        # the kernel indexes both tensors in 16-byte units with 32-bit integers
+        and params.n * params.groups * max(params.h * params.w, params.p * params.q) < 2**31
     )
 
 

@@ -208,3 +208,74 @@ def test_convnext_shaped_network_at_batch_128():
     assert float((got8 - want).abs().max()) < 0.08 * max(1.0, float(want.abs().max()))
     assert torch.equal(got8.argmax(dim=1), want.argmax(dim=1))
     assert torch.isfinite(got).all()
+
+
+def _repeat_images(t, rep):
+    """[n, C, H, W] -> [n * rep, C, H, W] on the GPU in channels_last memory, the n images repeated."""
+    nhwc = t.cuda().permute(0, 2, 3, 1).contiguous()
+    return nhwc.repeat(rep, 1, 1, 1).permute(0, 3, 1, 2)
+
+
+def _blocks_equal_first(t, rep):
+    v = t.permute(0, 2, 3, 1).reshape(rep, -1)
+    return all(bool((v[i:i + 64] == v[0:1]).all()) for i in range(0, rep, 64))
+
+
+@pytest.mark.parametrize("mode", ["1", "0"])
+def test_tensors_beyond_4_gib(monkeypatch, mode):
+    """N = 11000 images of 64 channels, 56x56: every activation tensor holds 2.2e9 elements in
+    4.4 GB, past what 32-bit element indices and byte offsets reach.  The batch is 8 seeded
+    images repeated 1375 times: the first and last 8 outputs and input gradients are checked
+    against the oracle, every other block of 8 must equal the first bit for bit, and the weight
+    and bias gradients must be 1375 times the oracle's for the 8 images.  With the fused backward
+    kernel and with the separate ones."""
+    monkeypatch.setenv("SPIO_FUSED_BACKWARD", mode)
+    rep = 1375
+    x, w, b, dy = oracle.make_args(8, 64, 56, 56, 3, 3, 1, 1, True, 5, weight_init="kaiming")
+    y_e = oracle.fprop_torch(x, w, b, 1, 1)
+    dx_e, dw_e, db_e = oracle.grads_torch(x, w, b, dy, 1, 1)
+    xb, dyb = _repeat_images(x, rep), _repeat_images(dy, rep)
+    assert xb.numel() > 2**31 and xb.is_contiguous(memory_format=torch.channels_last)
+    wg, bg = to_gpu(w), to_gpu(b)
+    y = conv2d_gw8(xb, wg, bg, stride=1, padding_y=1, padding_x=1, groups=8)
+    oracle.check_close(y[:8], y_e, what="fprop, first images")
+    oracle.check_close(y[-8:], y_e, what="fprop, last images")
+    assert _blocks_equal_first(y, rep)
+    del y
+    dx, dw, db = torch.ops.spio.conv2d_gw8_backward(xb, wg, bg, dyb, 1, 1, True, True, True)
+    oracle.check_close(dx[:8], dx_e, what="dgrad, first images")
+    oracle.check_close(dx[-8:], dx_e, what="dgrad, last images")
+    assert _blocks_equal_first(dx, rep)
+    for got, expected, name in ((dw, dw_e * rep, "grad_weight"), (db, db_e * rep, "grad_bias")):
+        err = (got.cpu().float() - expected).abs().max().item()
+        assert err <= 1e-3 * expected.abs().max().item(), f"{name}: {err}"
+
+
+def test_layernorm_tensors_beyond_4_gib():
+    """LayerNorm2d forward and backward on 11000 images of 96 channels, 56x56 (3.3e9 elements,
+    6.6 GB per tensor): 8 seeded images repeated; blocks equal the first one, the first block is
+    checked against torch in fp32, the channel sums are 1375 times those of the 8 images."""
+    from spio_amd.functional import layernorm_2d
+    from spio_amd.functional.layernorm_2d_function import layernorm_2d_backward
+
+    rep = 1375
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(8, 96, 56, 56, generator=g) * 2 + 0.5).half()
+    dy = torch.randn(8, 96, 56, 56, generator=g).half()
+    w, b = torch.randn(96, generator=g), torch.randn(96, generator=g)
+    xr = x.float().requires_grad_(True)
+    wr = w.clone().requires_grad_(True)
+    y_e = torch.nn.functional.layer_norm(xr.permute(0, 2, 3, 1), (96,), wr, b, 1e-6).permute(0, 3, 1, 2)
+    y_e.backward(dy.float())
+    xb, dyb = _repeat_images(x, rep), _repeat_images(dy, rep)
+    assert xb.numel() > 2**31
+    y = layernorm_2d(xb, w.cuda(), b.cuda(), 1e-6)
+    torch.testing.assert_close(y[:8].float().cpu(), y_e.detach(), rtol=2e-3, atol=4e-3)
+    assert _blocks_equal_first(y, rep)
+    del y
+    dx, sums = layernorm_2d_backward(xb, dyb, w.cuda(), 1e-6)
+    torch.testing.assert_close(dx[:8].float().cpu(), xr.grad, rtol=4e-3, atol=4e-3)
+    assert _blocks_equal_first(dx, rep)
+    sums = sums.cpu()
+    for got, expected in ((sums[0], wr.grad * rep), (sums[1], dy.float().sum(dim=(0, 2, 3)) * rep)):
+        assert (got - expected).abs().max().item() <= 1e-3 * expected.abs().max().item()

@@ -392,3 +392,24 @@ def test_counter_figures_in_profiles_were_measured_with_the_committed_kernel_sou
     m = bench.stream_model(18.3, 102769664)
     assert abs(m["stream_model_us"] - (2.2 + 102769664 / 6.2e6)) < 0.01 and 0.9 < m["frac_of_stream_model"] < 1.1
     assert re.fullmatch(r"[0-9a-f]{12}", bench.source_digest("conv2d_gw8_mfma.hip"))
+
+
+def test_weight_gradient_mfma_kernel_is_not_offered_past_its_32_bit_indices():
+    """The MFMA weight-gradient kernel indexes its tensors in 16-byte units with 32-bit integers:
+    up to 32 GiB per tensor.  Beyond that only the general kernel (64-bit arithmetic) is offered;
+    the forward and fused backward kernels rebase their descriptors per image block and stay."""
+    from spio_amd.hip.driver import DeviceAttributes
+    from spio_amd.kernels import (
+        Conv2dGw8Params,
+        conv2d_gw8_bgrad_kernel_factory,
+        conv2d_gw8_kernel_factory,
+        conv2d_gw8_wgrad_kernel_factory,
+    )
+
+    attr = DeviceAttributes()
+    fits = Conv2dGw8Params(n=11000, c=64, h=56, w=56)  # 4.4 GB per tensor
+    past = Conv2dGw8Params(n=90000, c=64, h=56, w=56)  # 36 GB per tensor
+    assert {c.variant for c in conv2d_gw8_wgrad_kernel_factory.configs(fits, attr)} >= {"mfma"}
+    assert {c.variant for c in conv2d_gw8_wgrad_kernel_factory.configs(past, attr)} == {"direct"}
+    assert conv2d_gw8_kernel_factory.configs(past, attr)[0].variant == "mfma"
+    assert conv2d_gw8_bgrad_kernel_factory.configs(past, attr)
