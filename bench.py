@@ -936,7 +936,7 @@ def precompile_recorded_kernels():
 
 
 def configs_block(args, device):
-    """Compact measurements of every BASELINE configuration next to the headline workload."""
+    """Compact measurements of every benchmark configuration (cfg1..cfg5) next to the headline workload."""
     import torch
 
     t0 = time.perf_counter()
